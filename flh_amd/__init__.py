@@ -48,7 +48,7 @@ class PackedQuantizedTensor:
         return self.quantized_x.dtype
 
 
-from . import functional, nn, cuda  # noqa: E402,F401
+from . import functional, nn, cuda, hql  # noqa: E402,F401
 
 
 def install_as_flh():

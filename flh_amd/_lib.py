@@ -28,7 +28,7 @@ _SIG = {
     "flh_gemm_i4_i32": (_c.c_int, [_PTR, _PTR, _PTR, _c.c_size_t, _c.c_size_t, _c.c_size_t, _PTR]),
     "flh_gemm_f6_o16_multi": (_c.c_int, [_PTR, _PTR, _c.c_int, _PTR, _PTR, _PTR, _PTR, _c.c_size_t, _c.c_size_t,
                                          _c.c_int, _c.c_int, _PTR]),
-    "flh_probe_mfma_i8": (_c.c_int, [_c.c_int, _c.c_int, _PTR]),
+    "flh_gemm_set_tuning": (_c.c_int, [_c.c_int, _c.c_int]),
     "flh_rotate_quant_gemm_i4_o16": (_c.c_int, [_PTR, _PTR, _PTR, _PTR, _c.c_size_t, _c.c_size_t, _c.c_size_t,
                                                 _c.c_int, _PTR]),
     "flh_encode_f6": (_c.c_int, [_PTR, _PTR, _c.c_size_t, _c.c_size_t, _PTR]),
@@ -57,6 +57,17 @@ _SIG = {
 }
 EXPORTS = tuple(_SIG)
 
+# The reference's C++-linkage declarations (include/flh_reference_native.h), by their Itanium-mangled names over
+# `__half`: what a binding file compiled for HIP links against.  Same argument lists as the C-linkage twins above.
+_SIG_CXX = {
+    "flhDenseLayerGEMM_i4_o16_gs": "_Z27flhDenseLayerGEMM_i4_o16_gsiPKhS0_P6__halfmmmPKS1_S4_",
+    "had_and_quant_host": "_Z18had_and_quant_hostPK6__halfPhPS_j",
+    "quant_and_pack_host": "_Z19quant_and_pack_hostPK6__halfPhPS_j",
+    "had_and_quant_host_gs": "_Z21had_and_quant_host_gsiPK6__halfPhPS_j",
+    "quant_and_pack_host_gs": "_Z22quant_and_pack_host_gsiPK6__halfPhPS_j",
+}
+EXPORTS_CXX = tuple(_SIG_CXX.values())
+
 
 class FLHLibraryError(RuntimeError):
     pass
@@ -77,6 +88,9 @@ def load():
         fn = getattr(lib, name)  # AttributeError if the library does not export it
         fn.restype = res
         fn.argtypes = args
+    for plain, mangled in _SIG_CXX.items():
+        fn = getattr(lib, mangled)
+        fn.restype, fn.argtypes = _SIG[plain]
     if lib.flh_abi_version() != 1:
         raise FLHLibraryError("libflh_hip.so has an unexpected ABI version; rebuild it")
     _lib = lib

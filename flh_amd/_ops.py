@@ -57,6 +57,8 @@ def _check_gemm_inputs(A, B, A_scale, B_scale):
            "tensors must be contiguous")
     _check(A.dim() == 2 and B.dim() == 2, "A/B must be 2D")
     _check(B.size(1) == A.size(1), "B.shape[1] must equal A.shape[1]")
+    _check(B.device == A.device and A_scale.device == A.device and B_scale.device == A.device,
+           "tensors must be on one device")
 
 
 def gemm_i4_dequant(A, B, A_scale, B_scale, group_size=128):
@@ -71,6 +73,8 @@ def _gemm_i4_dequant_checked(A, B, A_scale, B_scale, group_size):
     M, Kp = A.shape
     N, K = B.size(0), Kp * 2
     _check(A_scale.dim() == 2 and B_scale.dim() == 2, "scale must be 2D")
+    _check(A_scale.size(0) == M, "A_scale.shape[0] must equal M")
+    _check(B_scale.size(0) == N, "B_scale.shape[0] must equal N")
     _check(K % 128 == 0, "K must be a multiple of 128")
     D = torch.empty((M, N), dtype=torch.float16, device=A.device)
     if M == 0 or N == 0:
@@ -199,15 +203,9 @@ def rotate_quantize_gemm_i4_multi(x, Bs, B_scales):
     return Ds
 
 
-PROBE_MFMA_OPS_PER_ITERATION = 512 * 4 * 16 * 65536     # workgroups x waves x instructions x operations
-
-
-def probe_mfma_i8(pattern, iters):
-    """Diagnostic: one launch, on the current device and stream, of a loop of int8 matrix instructions on zeros (0),
-    int4 codes x 16 (1) or random bytes (2); PROBE_MFMA_OPS_PER_ITERATION * iters integer operations, to be timed
-    by the caller."""
-    dev = torch.device("cuda", torch.cuda.current_device())
-    _run("flh_probe_mfma_i8", dev, int(pattern), int(iters), torch.cuda.current_stream(dev).cuda_stream)
+def gemm_set_tuning(tile=0, k_split=0):
+    """Test / tuning hook: force the GEMM tile (64, 128, 256) and in-workgroup K split (1, 2, 4); 0 = automatic."""
+    _lib.check(_lib.load().flh_gemm_set_tuning(int(tile), int(k_split)))
 
 
 def encode_f6(packed):
@@ -244,6 +242,7 @@ def _check_f6(A6, B6):
     _check(A6.is_contiguous() and B6.is_contiguous(), "tensors must be contiguous")
     _check(A6.dim() == 2 and B6.dim() == 2 and A6.size(1) == B6.size(1) and A6.size(1) % 96 == 0,
            "encoded operands must be 2D with equal K")
+    _check(A6.device == B6.device, "tensors must be on one device")
     return A6.size(0), B6.size(0), A6.size(1) // 96 * 128
 
 
@@ -254,6 +253,7 @@ def gemm_f6_dequant_o16(A6, B6, A_scale, B_scale):
            "scales must be float16 CUDA tensors")
     _check(A_scale.is_contiguous() and B_scale.is_contiguous() and A_scale.numel() == M and B_scale.numel() == N,
            "one scale per row of A and of B expected")
+    _check(A_scale.device == A6.device and B_scale.device == A6.device, "tensors must be on one device")
     D = torch.empty((M, N), dtype=torch.float16, device=A6.device)
     if M and N:
         _run("flh_gemm_f6_o16", A6.device, A6.data_ptr(), B6.data_ptr(), A_scale.data_ptr(), B_scale.data_ptr(),
@@ -272,6 +272,7 @@ def gemm_f6_dequant_o16_gs(A6, B6, A_scale, B_scale):
            "scales must be contiguous and 2D")
     _check(A_scale.size(0) == M and A_scale.size(1) in (1, ng), "A_scale must be [M, K/128] or [M, 1]")
     _check(B_scale.size(0) == N and B_scale.size(1) == ng, "B_scale must be [N, K/128]")
+    _check(A_scale.device == A6.device and B_scale.device == A6.device, "tensors must be on one device")
     D = torch.empty((M, N), dtype=torch.float16, device=A6.device)
     if M and N:
         _run("flh_gemm_f6_o16_gs", A6.device, A6.data_ptr(), B6.data_ptr(), A_scale.data_ptr(), B_scale.data_ptr(),

@@ -307,10 +307,6 @@ __global__ __launch_bounds__(512) void rotate_quant_mfma_dense_kernel(const __ha
   extern __shared__ __align__(1024) h8 mfrag[];        // [kb][s][nt][lane], then the maxima
   float* red = (float*)(mfrag + NFRAG * 64);           // [parity][row slot][mt]
   const uint8_t* xs = (const uint8_t*)(red + 16);      // SPLIT: the row, DT * 32 rows of 128 bytes, chunk c of row j at c ^ (j & 7)
-#ifdef FLH_TRACE_DENSE
-  const long long T0 = __builtin_amdgcn_s_memtime();
-  long long trace_t[4];
-#endif
   const int lane = threadIdx.x & 63, col = lane & 31, h = lane >> 5;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int slot = wave >> 1, mt = wave & 1;
@@ -386,9 +382,6 @@ __global__ __launch_bounds__(512) void rotate_quant_mfma_dense_kernel(const __ha
 #pragma unroll
     for (int t = 0; t < NB - 1; ++t) load_tile(nullptr, t, t);
   }
-#ifdef FLH_TRACE_DENSE
-  trace_t[1] = __builtin_amdgcn_s_memtime();
-#endif
 
   // The wave pairs of row slots 2 and 3 run one phase behind those of slots 0 and 1: every iteration has two
   // workgroup barriers (after the MFMA phase, where a pair exchanges its maxima, and after the quantising
@@ -436,9 +429,6 @@ __global__ __launch_bounds__(512) void rotate_quant_mfma_dense_kernel(const __ha
             w[nt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(h8, a[s]), fr[f % RING], w[nt], 0, 0, 0);
         }
     }
-#ifdef FLH_TRACE_DENSE
-    trace_t[2] = __builtin_amdgcn_s_memtime();
-#endif
     if constexpr (!SPLIT) {
       if (base + stride < M) {                         // the next row's first tiles travel during the epilogue
 #pragma unroll
@@ -455,13 +445,7 @@ __global__ __launch_bounds__(512) void rotate_quant_mfma_dense_kernel(const __ha
         mx = __builtin_fmaxf(__builtin_fmaxf(__builtin_fabsf(w[nt][2 * u]), __builtin_fabsf(w[nt][2 * u + 1])), mx);
     mx = wave_max(mx);
     if (lane == 0) red[(parity * 4 + slot) * 2 + mt] = mx;
-#ifdef FLH_TRACE_DENSE
-    const long long t_max = __builtin_amdgcn_s_memtime();
-#endif
     __syncthreads();                                   // the pair's maxima (slots alternate between rows)
-#ifdef FLH_TRACE_DENSE
-    const long long t_bar = __builtin_amdgcn_s_memtime();
-#endif
     if constexpr (SPLIT) {
       mx = 0.f;
 #pragma unroll
@@ -495,11 +479,6 @@ __global__ __launch_bounds__(512) void rotate_quant_mfma_dense_kernel(const __ha
     if (careful) emit(std::true_type{});
     else emit(std::false_type{});
     if (valid && lane == 0 && mt == 0 && (!SPLIT || slot == 0)) scales[row] = __builtin_bit_cast(__half, s16);
-#ifdef FLH_TRACE_DENSE
-    trace_t[3] = __builtin_amdgcn_s_memtime();
-    if (valid && lane == 0 && mt == 0) { long long* tq = (long long*)(q + (size_t)row * (K / 2)); tq[0] = t_max - trace_t[2]; tq[1] = trace_t[2] - trace_t[1]; tq[2] = t_bar - t_max; tq[3] = trace_t[3] - t_bar; }
-    trace_t[1] = trace_t[3];
-#endif
     barrier_no_fence();                                // end of the quantising phase (see above the loop)
     if constexpr (SPLIT) break;                        // one row per workgroup: only that row was staged
   }

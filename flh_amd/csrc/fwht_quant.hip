@@ -754,21 +754,6 @@ extern "C" int flh_fwht_f16_inplace(flh_half* x, uint32_t R, int group, void* st
   return group_dispatch(nullptr, nullptr, nullptr, (__half*)x, R, group, true, false, 1.0f, (hipStream_t)stream);
 }
 
-extern "C" void had_and_quant_host(const flh_half* data, uint8_t* quantized, flh_half* scales, uint32_t M) {
-  (void)flh_group_quant_i4(data, quantized, scales, M, 128, 1, 1.0f, nullptr);
-}
-extern "C" void quant_and_pack_host(const flh_half* data, uint8_t* quantized, flh_half* scales, uint32_t M) {
-  (void)flh_group_quant_i4(data, quantized, scales, M, 128, 0, 1.0f, nullptr);
-}
-extern "C" void had_and_quant_host_gs(int group_size, const flh_half* data, uint8_t* quantized, flh_half* scales,
-                                      uint32_t M) {
-  (void)flh_group_quant_i4(data, quantized, scales, M, group_size, 1, 1.0f, nullptr);
-}
-extern "C" void quant_and_pack_host_gs(int group_size, const flh_half* data, uint8_t* quantized, flh_half* scales,
-                                       uint32_t M) {
-  (void)flh_group_quant_i4(data, quantized, scales, M, group_size, 0, 1.0f, nullptr);
-}
-
 extern "C" int flh_rotate_quant_i4(const flh_half* x, uint8_t* q_packed, flh_half* scales, flh_half* y_out, uint32_t M,
                                    uint32_t K, int hadamard, int had_group, int scale_group, float clip_ratio,
                                    void* stream) {

@@ -27,7 +27,6 @@
 // sits in slot 6 r + (c ^ ((r >> 3) & 1)): sixteen consecutive rows read at one logical chunk touch sixteen
 // different groups of four banks.  Fragment reads run half a stage ahead of the MFMAs that use them.
 #include <atomic>
-#include <stdlib.h>
 
 #include <type_traits>
 
@@ -419,11 +418,10 @@ int launch_f6_grouped(const GemmArgs& a, hipStream_t stream) {
   return launch_f6<64, 64, 32, 32, 3, EPI>(a, stream);
 }
 
-// FLH_GEMM_TILE (256 / 128 / 64) overrides the tile choice (tuning aid, used by the tests to cover every variant)
+// flh_gemm_set_tuning overrides the tile choice (256 / 128 / 64; the hook through which the tests cover every variant)
 template <int EPI>
 int launch_f6_by_shape(const GemmArgs& a, hipStream_t stream) {
-  const char* e_tile = getenv("FLH_GEMM_TILE");
-  const int env_tile = e_tile ? atoi(e_tile) : 0;
+  const int env_tile = g_tune_tile.load(std::memory_order_relaxed);
   const int n_all = total_n_f6(a);
   auto tiles = [&](int bm, int bn) { return (long)((a.M + bm - 1) / bm) * ((n_all + bn - 1) / bn); };
   // measured at M = 2048 on the Llama shapes: two 128 x 128 workgroups per compute unit beat one 256 x 128

@@ -1,5 +1,7 @@
 // Shared declarations of the int4 GEMM translation units.
 #pragma once
+#include <atomic>
+
 #include "common.h"
 
 namespace flh {
@@ -8,6 +10,9 @@ namespace flh {
 enum Epilogue { kRowScale = 0, kGroupScale = 1, kInt32 = 2, kTokenGroup = 3 };
 
 constexpr int kMaxGemmSegments = 4;
+
+// tile / K-split override of the shape heuristics (0 = automatic), set by flh_gemm_set_tuning
+extern std::atomic<int> g_tune_tile, g_tune_ks;
 
 struct GemmArgs {
   const uint8_t* A;     // [M, K/2] packed activations
@@ -26,9 +31,6 @@ struct GemmArgs {
   const uint8_t* seg_B[kMaxGemmSegments];
   const __half* seg_Bs[kMaxGemmSegments];
   void* seg_D[kMaxGemmSegments];
-#ifdef FLH_GEMM_TRACE
-  long long* trace;
-#endif
 };
 
 // Small-M (decode) kernels: weight-streaming, split over K inside a workgroup.

@@ -28,13 +28,15 @@
 // and four consecutive columns n per register quad, which packs into 8-byte LDS writes for
 // the epilogue; the tile leaves through LDS as full 128-byte row segments.
 #include <atomic>
-#include <stdlib.h>
 
 #include <type_traits>
 
 #include "gemm_i4.h"
 
 namespace flh {
+
+// tile / K-split override of the shape heuristics (0 = automatic), set by flh_gemm_set_tuning
+std::atomic<int> g_tune_tile{0}, g_tune_ks{0};
 
 namespace {
 
@@ -44,11 +46,6 @@ namespace {
 constexpr int kStageBytes = 64;   // packed bytes of K per row per stage (128 codes)
 constexpr int kEpiPad = 16;       // bytes of padding per row of the epilogue staging tile
 
-#ifdef FLH_GEMM_TRACE
-#define TRACE(slot) do { if (tid == 0) p.trace[blockIdx.x * 16 + (slot)] = __builtin_amdgcn_s_memtime(); } while (0)
-#else
-#define TRACE(slot) do { } while (0)
-#endif
 
 __device__ __forceinline__ void unpack8(const v4i w, v4i& lo, v4i& hi) {
 #pragma unroll
@@ -111,14 +108,6 @@ void gemm_i4_kernel(const GemmArgs p) {
   extern __shared__ __align__(1024) uint8_t lds[];    // [KS][STAGES][STAGE]
 
   const int tid = threadIdx.x;
-  TRACE(0);
-#ifdef FLH_GEMM_TRACE
-  if (tid == 0) {
-    p.trace[blockIdx.x * 16 + 8] = __builtin_amdgcn_s_memrealtime();
-    p.trace[blockIdx.x * 16 + 10] = __builtin_amdgcn_s_getreg(4 | (31 << 11));
-    p.trace[blockIdx.x * 16 + 11] = __builtin_amdgcn_s_getreg(20 | (31 << 11));
-  }
-#endif
   const int lane = tid & 63;
   const int wave_all = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int quad = KS == 1 ? 0 : wave_all / WPQ;      // which slice of K
@@ -332,28 +321,14 @@ void gemm_i4_kernel(const GemmArgs p) {
     unpack8(pk[f], ulo[0][f], uhi[0][f]);
     pk[f] = *frag_ptr(0, f, off_k1);
   }
-  TRACE(1);
 
-#ifdef FLH_GEMM_TRACE
-  long long trace_vm = 0, trace_bar = 0;
-#endif
   int stage = 0;
   for (int kt = 0; kt < KTmax; ++kt) {
     const int nxt = stage + 1 == STAGES ? 0 : stage + 1;
-#ifdef FLH_GEMM_TRACE
-    const long long tw0 = __builtin_amdgcn_s_memtime();
-#endif
     wait_vmcnt<(STAGES - 3) * NI>();                  // this wave's part of stage kt+1 has landed
-#ifdef FLH_GEMM_TRACE
-    const long long tw1 = __builtin_amdgcn_s_memtime();
-#endif
     // ... everybody's has, and stage kt-1 is free: its last fragment reads were consumed an iteration ago;
     // the LDS reads still in flight here belong to stage kt, which nobody overwrites before the next barrier
     barrier_no_fence();
-#ifdef FLH_GEMM_TRACE
-    trace_vm += tw1 - tw0;
-    trace_bar += __builtin_amdgcn_s_memtime() - tw1;
-#endif
     if constexpr (GROUPED) {
       // the next block of eight group scales, requested at the end of the previous iteration
       if (kt % SPB == SPB - 1) sc_store(kt / SPB + 1);
@@ -400,13 +375,8 @@ void gemm_i4_kernel(const GemmArgs p) {
     }
     stage = nxt;
   }
-  TRACE(2);
-#ifdef FLH_GEMM_TRACE
-  if (tid == 0) { p.trace[blockIdx.x * 16 + 6] = trace_vm; p.trace[blockIdx.x * 16 + 7] = trace_bar; }
-#endif
   wait_vmcnt<0>();                                    // drain the trailing reloads
   __syncthreads();                                    // every wave is done with the ring
-  TRACE(3);
 
   // ---- K split: add the quads' accumulators through LDS -------------------------------
   int rb = 0;                                         // first 32-row block of the wave tile this quad finishes
@@ -541,7 +511,6 @@ void gemm_i4_kernel(const GemmArgs p) {
           *(h4*)(ep + (i * 32 + frag_row) * EPI_PITCH + nl * 2) = v;
         }
       }
-    TRACE(4);
     // ... and write it out as whole row segments (the tile is private to the wave: no barrier)
     constexpr int CPR = WN / 8;                        // 16-byte chunks per row of the wave tile
     constexpr int RPI = 64 / CPR;                      // rows per store instruction
@@ -565,10 +534,6 @@ void gemm_i4_kernel(const GemmArgs p) {
       }
     }
   }
-  TRACE(5);
-#ifdef FLH_GEMM_TRACE
-  if (tid == 0) p.trace[blockIdx.x * 16 + 9] = __builtin_amdgcn_s_memrealtime();
-#endif
 }
 
 // output columns of a launch over all its weight matrices
@@ -608,13 +573,11 @@ int launch(GemmArgs a, hipStream_t stream) {
 // Tile and K-split choice for the one-scale-per-row and int32 epilogues: the largest tile that
 // still gives every compute unit a workgroup (else the smallest), and for the smallest tile with
 // at most two workgroups per compute unit, a K split that puts more waves on every SIMD.
-// FLH_GEMM_TILE (256 / 128 / 64) and FLH_GEMM_KS (1 / 2 / 4) override the choice; they are read on every call, which
-// is how the tests reach every variant from one process (two getenv calls against a launch of microseconds).
+// flh_gemm_set_tuning(tile, ks) overrides the choice process-wide (0 = automatic): the hook through which the
+// tests reach every variant and a tuning run compares them.
 template <int EPI>
 int launch_by_shape(const GemmArgs& a, hipStream_t stream) {
-  const char* e_tile = getenv("FLH_GEMM_TILE");
-  const char* e_ks = getenv("FLH_GEMM_KS");
-  const int env_tile = e_tile ? atoi(e_tile) : 0, env_ks = e_ks ? atoi(e_ks) : 0;
+  const int env_tile = g_tune_tile.load(std::memory_order_relaxed), env_ks = g_tune_ks.load(std::memory_order_relaxed);
   const int n_all = total_n(a);
   auto tiles = [&](int bm, int bn) { return (long)((a.M + bm - 1) / bm) * ((n_all + bn - 1) / bn); };
   const int kt = a.K >> 7;
@@ -689,10 +652,14 @@ int check_common(const void* A, const void* B, const void* D, size_t M, size_t N
 
 using namespace flh;
 
-#ifdef FLH_GEMM_TRACE
-static long long* flh_gemm_trace_buffer = nullptr;
-extern "C" void flh_gemm_set_trace(long long* p) { flh_gemm_trace_buffer = p; }
-#endif
+
+extern "C" int flh_gemm_set_tuning(int tile, int k_split) {
+  if ((tile != 0 && tile != 64 && tile != 128 && tile != 256) || (k_split != 0 && k_split != 1 && k_split != 2 && k_split != 4))
+    return fail(FLH_EINVAL, "gemm tuning: tile must be 0, 64, 128 or 256 and k_split 0, 1, 2 or 4");
+  g_tune_tile.store(tile, std::memory_order_relaxed);
+  g_tune_ks.store(k_split, std::memory_order_relaxed);
+  return FLH_OK;
+}
 
 extern "C" int flh_gemm_i4_o16(const uint8_t* A, const uint8_t* B, const flh_half* a_scale, const flh_half* b_scale,
                                flh_half* D, size_t M, size_t N, size_t K, int a_cols, int b_cols, int group,
@@ -709,9 +676,6 @@ extern "C" int flh_gemm_i4_o16(const uint8_t* A, const uint8_t* B, const flh_hal
       return fail(FLH_EINVAL, "gemm: scale columns (%d, %d) must be 1 or K/group = %d", a_cols, b_cols, ng);
   }
   GemmArgs g{A, B, (const __half*)a_scale, (const __half*)b_scale, D, (int)M, (int)N, (int)K, a_cols, b_cols, 0, 0, 0};
-#ifdef FLH_GEMM_TRACE
-  g.trace = flh_gemm_trace_buffer;
-#endif
   return gemm_dispatch(g, grouped ? kGroupScale : kRowScale, group, (hipStream_t)stream);
 }
 
@@ -748,9 +712,6 @@ extern "C" int flh_gemm_i4_o16_multi(const uint8_t* A, const flh_half* a_scale, 
     g.seg_D[s] = D[s];
     g.seg_N[s] = (int)N[s];
   }
-#ifdef FLH_GEMM_TRACE
-  g.trace = flh_gemm_trace_buffer;
-#endif
   return gemm_dispatch(g, grouped ? kGroupScale : kRowScale, group, (hipStream_t)stream);
 }
 
@@ -758,20 +719,5 @@ extern "C" int flh_gemm_i4_i32(const uint8_t* A, const uint8_t* B, int32_t* C, s
                                void* stream) {
   if (int e = check_common(A, B, C, M, N, K)) return e;
   GemmArgs g{A, B, nullptr, nullptr, C, (int)M, (int)N, (int)K, 1, 1, 0, 0, 0};
-#ifdef FLH_GEMM_TRACE
-  g.trace = flh_gemm_trace_buffer;
-#endif
   return gemm_dispatch(g, kInt32, 0, (hipStream_t)stream);
-}
-
-extern "C" void flhDenseLayerGEMM_i4_o16(const uint8_t* A, const uint8_t* B, const flh_half* A_scale,
-                                         const flh_half* B_scale, flh_half* D, size_t M, size_t N, size_t K) {
-  const int ng = (int)(K / 128);
-  (void)flh_gemm_i4_o16(A, B, A_scale, B_scale, D, M, N, K, ng, ng, 128, nullptr);
-}
-
-extern "C" void flhDenseLayerGEMM_i4_o16_gs(int group_size, const uint8_t* A, const uint8_t* B, flh_half* D, size_t M,
-                                            size_t N, size_t K, const flh_half* A_scale, const flh_half* B_scale) {
-  const int ng = group_size > 0 ? (int)(K / group_size) : 0;
-  (void)flh_gemm_i4_o16(A, B, A_scale, B_scale, D, M, N, K, ng, ng, group_size, nullptr);
 }

@@ -33,14 +33,23 @@ class LinearFLH(torch.nn.Module):
         else:
             self.bias = None
         # Opt-in (extension): run prefill-sized calls on the 6-bit matrix instruction.  The weights are then held a
-        # second time, re-encoded at 6 bits per code (built on first use, dropped by `drop_six_bit_weights()` after
-        # the packed weights change); outputs are bit-identical.  Pays for wide layers and group scales.
+        # second time, re-encoded at 6 bits per code; outputs are bit-identical.  Pays for wide layers and group scales.
+        # The encoding is rebuilt whenever `w_packed` has been written to or replaced (in-place copies, load_state_dict,
+        # .to(device)): it is keyed on the buffer's storage address and version counter.
         self.six_bit = False
         self.six_bit_min_rows = 256
         self._w6 = None
+        self._w6_key = None
 
     def drop_six_bit_weights(self):
-        self._w6 = None
+        self._w6 = self._w6_key = None
+
+    def _six_bit_weights(self):
+        key = (self.w_packed.data_ptr(), self.w_packed._version, self.w_packed.device)
+        if self._w6 is None or self._w6_key != key:
+            self._w6 = _pkg._CUDA.encode_f6(self.w_packed.view(self.out_features, self.in_features // 2))
+            self._w6_key = key
+        return self._w6
 
     def _six_bit_applies(self, rows, a_scale, w_scale, group):
         if not (self.six_bit and rows.is_cuda and rows.size(0) >= self.six_bit_min_rows and self.in_features % 128 == 0):
@@ -61,16 +70,15 @@ class LinearFLH(torch.nn.Module):
         encoded = rows.size(1) * 4 == self.in_features * 3      # activations already in the 6-bit format
         if encoded or self._six_bit_applies(rows, a_rows, w_scale, group):
             ops = _pkg._CUDA
-            if self._w6 is None:
-                self._w6 = ops.encode_f6(self.w_packed.view(self.out_features, self.in_features // 2))
+            w6 = self._six_bit_weights()
             a6 = rows.contiguous() if encoded else ops.encode_f6(rows.contiguous())
             if encoded and not ((w_scale.size(1) == 1 and a_rows.size(1) == 1) or
                                 (group == 128 and w_scale.size(1) == self.in_features // 128)):
                 raise ValueError("6-bit activations need per-token x per-channel scales or group-of-128 weight scales")
             if w_scale.size(1) == 1:
-                y = ops.gemm_f6_dequant_o16(a6, self._w6, a_rows.contiguous(), w_scale)
+                y = ops.gemm_f6_dequant_o16(a6, w6, a_rows.contiguous(), w_scale)
             else:
-                y = ops.gemm_f6_dequant_o16_gs(a6, self._w6, a_rows.contiguous(), w_scale)
+                y = ops.gemm_f6_dequant_o16_gs(a6, w6, a_rows.contiguous(), w_scale)
             if self.bias is not None:
                 y = y + self.bias
             return y.view(*lead, self.out_features)
@@ -98,11 +106,8 @@ class LinearFLH(torch.nn.Module):
         encoded = rows.size(1) * 4 == first.in_features * 3      # activations already in the 6-bit format
         if encoded or all(l._six_bit_applies(rows, a_rows, ws, group) for l, ws in zip(layers, w_scales)):
             # every layer opted into the 6-bit matrix instruction: one launch there as well
-            for l in layers:
-                if l._w6 is None:
-                    l._w6 = ops.encode_f6(l.w_packed.view(l.out_features, l.in_features // 2))
             a6 = rows.contiguous() if encoded else ops.encode_f6(rows.contiguous())
-            ys = ops.gemm_f6_dequant_multi(a6, [l._w6 for l in layers], a_rows.contiguous(), w_scales)
+            ys = ops.gemm_f6_dequant_multi(a6, [l._six_bit_weights() for l in layers], a_rows.contiguous(), w_scales)
         else:
             ys = ops.gemm_i4_dequant_multi(rows, [l.w_packed.view(l.out_features, l.in_features // 2) for l in layers],
                                            a_rows, w_scales, group)

@@ -1,28 +1,35 @@
 """One W4A4 Llama decoder layer on this library's kernels.
 
 The data path of the reference's FLH_LlamaAttention / FLH_LlamaMLP inside a LlamaDecoderLayer
-(flh/quantized_model/modeling_llama.py:312-526; norms :655-656): every linear is a LinearFLH fed by a group
-quantiser without online rotation (the reference folds its rotations into the weights and the embedding),
+(flh/quantized_model/modeling_llama.py:374-470 attention with cache, :522-526 MLP; norms :655-656): every linear is
+a LinearFLH fed by a quantiser,
 
     x -> RMSNorm -> quantiser -> q / k / v -> RoPE -> attention -> quantiser -> o_proj -> + x
       -> RMSNorm -> quantiser -> gate / up -> silu(gate) * up -> quantiser -> down_proj -> +
 
-with torch's scaled_dot_product_attention in place of the flash-attn package and a plain tensor pair as the
-key / value cache.  `fused=True` replaces "RMSNorm, quantiser" by RMSNormQuant, the projections that share an
-input by one launch (LinearFLH.forward_many) and "silu * up, quantiser" by SiluMulQuant: the same bits as the
-module-by-module sequence, which `fused=False` keeps for comparison.
+with torch's scaled_dot_product_attention in place of the flash-attn package.  The key / value cache is either a
+plain tensor pair that grows by concatenation (prefill, tests) or one layer of a preallocated StaticKVCache
+(decode steps that are captured into a graph).
 
-`activation="token"` is the other configuration of the path: every linear input is rotated as a whole row online
-(normalised Hadamard of 4096, resp. 172 x 64 for down_proj) and quantised with one scale per token, the weights are
-rotated the same way offline and carry one scale per output channel -- the arrangement of the reference's linear
-benchmarks (benchmark/nn/benchmark_linear_flh.py:139-222), put into the same layer.  There `fused=True` means RMSNorm
-inside the rotation kernel and shared-input launches.
+`activation="group"` is the arrangement of the reference's quantised model: group quantisers of 128 without online
+rotation (the rotations are folded into the weights and the embedding there) and group-scaled weights.
+`fused=True` replaces "RMSNorm, quantiser" by one launch, the projections that share an input by one launch
+(LinearFLH.forward_many) and "silu * up, quantiser" by one launch: the same bits as the module-by-module sequence,
+which `fused=False` keeps for comparison.
 
-Model loading, the tokenizer, sampling and the language-model head are the caller's.
+`activation="token"` is the path's other configuration: every linear input is rotated as a whole row online
+(normalised Hadamard of the hidden size; 172 x 64 resp. 28 x 512 for down_proj) and quantised with one scale per
+token; the weights are rotated the same way offline and carry one scale per output channel
+(`weight_group_size <= 0`, the arrangement of benchmark/nn/benchmark_linear_flh.py:139-222) or per group of 128
+input channels (the Llama-3 configuration).  There `fused=True` means RMSNorm inside the rotation kernel, shared-input
+launches and, for one or two tokens, the o_proj quantiser inside its GEMM.
+
+`record`: when set to a dict, every quantiser's input / codes / scales and every linear's output of the next call
+are stored in it (by stage name) -- the taps the parity tests compare with the CPU oracle stage by stage.
 """
 import torch
 
-from ..nn.fused import RMSNormQuant, SiluMulQuant
+from ..nn.fused import SiluMulQuant
 from ..nn.linear import LinearFLH
 from ..nn.normalization import RMSNorm
 from ..nn.quantization import ActQuantizer
@@ -39,6 +46,32 @@ def rotary_tables(positions, head_dim, theta=10000.0, dtype=torch.float16):
 def _rotate_half(x):
     half = x.size(-1) // 2
     return torch.cat((-x[..., half:], x[..., :half]), dim=-1)
+
+
+class StaticKVCache:
+    """Preallocated fp16 keys / values [layers][batch, kv_heads, max_len, head_dim].  `layer(i)` is what a decoder layer
+    takes as `kv_cache`: new keys / values are written in place at `positions` (a device index tensor, so a captured
+    graph can be replayed for other positions by overwriting it) and attention reads the first `kv_len` slots."""
+
+    def __init__(self, layers, batch, kv_heads, max_len, head_dim, device, dtype=torch.float16):
+        self.keys = [torch.zeros(batch, kv_heads, max_len, head_dim, dtype=dtype, device=device) for _ in range(layers)]
+        self.values = [torch.zeros_like(k) for k in self.keys]
+        self.max_len = max_len
+        self.kv_len = 0
+
+    class _Layer:
+        def __init__(self, owner, index):
+            self.owner, self.index = owner, index
+
+        def update(self, k, v, positions):
+            keys, values = self.owner.keys[self.index], self.owner.values[self.index]
+            keys.index_copy_(2, positions, k)
+            values.index_copy_(2, positions, v)
+            n = self.owner.kv_len
+            return keys[:, :, :n], values[:, :, :n]
+
+    def layer(self, index):
+        return StaticKVCache._Layer(self, index)
 
 
 class W4A4DecoderLayer(torch.nn.Module):
@@ -58,13 +91,16 @@ class W4A4DecoderLayer(torch.nn.Module):
         self.head_dim = hidden_size // num_heads
         self.intermediate_size, self.eps, self.fused = intermediate_size, eps, fused
         self.act_group_size = act_group_size
+        self.weight_group_size = weight_group_size
+        self.record = None
         kv = num_kv_heads * self.head_dim
         shapes = {"q_proj": (hidden_size, hidden_size), "k_proj": (hidden_size, kv), "v_proj": (hidden_size, kv),
                   "o_proj": (hidden_size, hidden_size), "gate_proj": (hidden_size, intermediate_size),
                   "up_proj": (hidden_size, intermediate_size), "down_proj": (intermediate_size, hidden_size)}
         for name, (k, n) in shapes.items():
+            g = weight_group_size if weight_group_size and weight_group_size > 0 else k
             setattr(self, name, LinearFLH(k, n, bias=False, device=device, in_group_size=act_group_size,
-                                          group_size=weight_group_size, no_hadamard=True))
+                                          group_size=g, no_hadamard=True))
         self.input_layernorm = RMSNorm(hidden_size, eps)
         self.post_attention_layernorm = RMSNorm(hidden_size, eps)
 
@@ -73,29 +109,34 @@ class W4A4DecoderLayer(torch.nn.Module):
         self.attn_quantizer1, self.attn_quantizer2 = quantiser(), quantiser()
         self.mlp_quantizer1, self.mlp_quantizer2 = quantiser(), quantiser()
         self._silu_mul_quant = SiluMulQuant(act_group_size)
+        self._norm16 = {}     # fp16 copies of the norm weights for the fused kernels: name -> (version, tensor)
 
     @classmethod
-    def from_float(cls, weights, num_heads, num_kv_heads, eps=1e-5, act_group_size=128, weight_group_size=128,
+    def from_float(cls, weights, num_heads, num_kv_heads, eps=1e-5, act_group_size=128, weight_group_size=None,
                    fused=True, activation="group", six_bit=False):
         """weights: fp16 tensors `q_proj` ... `down_proj` [N, K] (as nn.Linear stores them) and optionally
-        `input_layernorm` / `post_attention_layernorm` [hidden]; quantised round-to-nearest without rotation."""
+        `input_layernorm` / `post_attention_layernorm` [hidden]; quantised round-to-nearest ("group": as they are,
+        "token": after the rotation of their input side).  weight_group_size: None = 128 for "group" and one scale
+        per output channel for "token"; 128 with "token" is the Llama-3 arrangement; <= 0 one scale per channel."""
         hidden, inter = weights["q_proj"].size(1), weights["gate_proj"].size(0)
         device = weights["q_proj"].device
+        if weight_group_size is None:
+            weight_group_size = 128 if activation == "group" else 0
         layer = cls(hidden, num_heads, num_kv_heads, inter, eps, act_group_size, weight_group_size, fused, device,
                     activation)
         for name in cls.PROJECTIONS:
             w = weights[name]
+            lin = getattr(layer, name)
             if activation == "token":
-                # rows rotated by the same orthogonal transform as the activations, one scale per output channel
-                q, s = _ops().rotate_and_quantize_i4(w.to(torch.float16).contiguous(), hadamard="exact")
-                lin = LinearFLH(w.size(1), w.size(0), bias=False, device=device, group_size=w.size(1), no_hadamard=True)
+                # rows rotated by the same orthogonal transform as the activations
+                g = lin.weight_group_size if lin.weight_group_size < w.size(1) else 0
+                q, s = _ops().rotate_and_quantize_i4(w.to(torch.float16).contiguous(), hadamard="exact", scale_group=g)
                 lin.w_packed.copy_(q.reshape(-1))
-                lin.w_scale.copy_(s)
-                setattr(layer, name, lin)
+                lin.w_scale.copy_(s.reshape(lin.w_scale.shape))
                 continue
-            lin = torch.nn.Linear(w.size(1), w.size(0), bias=False, device=device, dtype=w.dtype)
-            lin.weight.data.copy_(w)
-            setattr(layer, name, LinearFLH.from_float(lin, weight_group_size=weight_group_size,
+            src = torch.nn.Linear(w.size(1), w.size(0), bias=False, device=device, dtype=w.dtype)
+            src.weight.data.copy_(w)
+            setattr(layer, name, LinearFLH.from_float(src, weight_group_size=weight_group_size,
                                                       in_group_size=act_group_size, no_hadamard=True))
         if six_bit:        # prefill-sized calls run on the 6-bit matrix instruction (second encoding of the weights)
             for name in cls.PROJECTIONS:
@@ -107,70 +148,118 @@ class W4A4DecoderLayer(torch.nn.Module):
         return layer
 
     # ------------------------------------------------------------------ pieces
-    def _token_quant(self, x, norm=None):
+    def _tap(self, name, value):
+        if self.record is not None:
+            self.record[name] = value
+
+    def _norm_weight16(self, name, norm):
+        """The norm weight as the fused kernels take it (fp16; exact for weights that came from an fp16 checkpoint),
+        converted once per version of the parameter."""
+        w = norm.weight
+        key = (w.data_ptr(), w._version)
+        hit = self._norm16.get(name)
+        if hit is None or hit[0] != key:
+            hit = (key, w.detach().to(torch.float16).contiguous())
+            self._norm16[name] = hit
+        return hit[1]
+
+    def _token_quant(self, stage, x, norm=None, norm_name=None):
         """Whole-row rotation + one scale per token (after RMSNorm when `norm` is given)."""
         rows = x.reshape(-1, x.size(-1)).contiguous()
         if norm is not None and self.fused:
-            q, s = _ops().rmsnorm_rotate_and_quantize_i4(rows, norm.weight.detach().to(torch.float16).contiguous(), norm.eps)
+            q, s = _ops().rmsnorm_rotate_and_quantize_i4(rows, self._norm_weight16(norm_name, norm), norm.eps)
         else:
             q, s = _ops().rotate_and_quantize_i4(norm(rows) if norm is not None else rows, hadamard=True)
+        self._tap(stage + ".input", rows)
+        self._tap(stage + ".codes", q)
+        self._tap(stage + ".scales", s)
         return s.view(*x.shape[:-1], 1), None, q.view(*x.shape[:-1], -1)
 
-    def _norm_quant(self, norm, quantizer, x):
+    def _norm_quant(self, stage, norm, norm_name, quantizer, x):
         if self.activation == "token":
-            return self._token_quant(x, norm)
+            return self._token_quant(stage, x, norm, norm_name)
         if self.fused:
             q, s = _ops().rmsnorm_and_quantize_i4_gs(x.reshape(-1, x.size(-1)).contiguous(),
-                                                     norm.weight.detach().to(torch.float16).contiguous(), norm.eps,
+                                                     self._norm_weight16(norm_name, norm), norm.eps,
                                                      self.act_group_size, False)
-            return s.view(*x.shape[:-1], -1), None, q.view(*x.shape[:-1], -1)
-        return quantizer(norm(x))
+            s, z, q = s.view(*x.shape[:-1], -1), None, q.view(*x.shape[:-1], -1)
+        else:
+            s, z, q = quantizer(norm(x))
+        self._tap(stage + ".input", x.reshape(-1, x.size(-1)))
+        self._tap(stage + ".codes", q.reshape(-1, q.size(-1)))
+        self._tap(stage + ".scales", s.reshape(-1, s.size(-1)))
+        return s, z, q
 
     def _project(self, layers, q, s, z):
         if self.fused:
             return LinearFLH.forward_many(layers, q, s)
         return [layer(q, s, z, x_is_packed=True) for layer in layers]
 
-    def attention(self, x, cos, sin, kv_cache=None):
+    def attention(self, x, cos, sin, kv_cache=None, positions=None):
         """x [B, T, hidden] fp16 (already the residual stream); cos / sin [T, head_dim] of the T new positions;
-        kv_cache: None or (keys, values) [B, kv_heads, past, head_dim].  Causal over past + T positions."""
+        kv_cache: None, a pair (keys, values) [B, kv_heads, past, head_dim] that grows by concatenation, or one layer
+        of a StaticKVCache together with `positions` (device int64 [T]: the slots the new tokens take; the cache's
+        kv_len says how many slots attention reads).  Causal over past + T positions."""
         b, t, _ = x.shape
-        s, z, q = self._norm_quant(self.input_layernorm, self.attn_quantizer1, x)
+        s, z, q = self._norm_quant("attn_in", self.input_layernorm, "input_layernorm", self.attn_quantizer1, x)
         qs, ks, vs = self._project([self.q_proj, self.k_proj, self.v_proj], q, s, z)
+        self._tap("q_proj", qs), self._tap("k_proj", ks), self._tap("v_proj", vs)
         qs = qs.view(b, t, self.num_heads, self.head_dim).transpose(1, 2)
         ks = ks.view(b, t, self.num_kv_heads, self.head_dim).transpose(1, 2)
         vs = vs.view(b, t, self.num_kv_heads, self.head_dim).transpose(1, 2)
         qs = qs * cos + _rotate_half(qs) * sin
         ks = ks * cos + _rotate_half(ks) * sin
-        if kv_cache is not None:
-            ks, vs = torch.cat((kv_cache[0], ks), dim=2), torch.cat((kv_cache[1], vs), dim=2)
-        cache = (ks, vs)
-        rep = self.num_heads // self.num_kv_heads
-        if rep > 1:
-            ks, vs = ks.repeat_interleave(rep, dim=1), vs.repeat_interleave(rep, dim=1)
+        static = isinstance(kv_cache, StaticKVCache._Layer)
+        if static:
+            ks, vs = kv_cache.update(ks, vs, positions)
+            cache = kv_cache
+        else:
+            if kv_cache is not None:
+                ks, vs = torch.cat((kv_cache[0], ks), dim=2), torch.cat((kv_cache[1], vs), dim=2)
+            cache = (ks, vs)
+        gqa = self.num_heads != self.num_kv_heads
         past = ks.size(2) - t
         if past == 0:
-            out = torch.nn.functional.scaled_dot_product_attention(qs, ks, vs, is_causal=t > 1)
+            out = torch.nn.functional.scaled_dot_product_attention(qs, ks, vs, is_causal=t > 1, enable_gqa=gqa)
+        elif t == 1:      # one new token sees every cached position
+            out = torch.nn.functional.scaled_dot_product_attention(qs, ks, vs, enable_gqa=gqa)
         else:
             mask = torch.ones(t, past + t, dtype=torch.bool, device=x.device).tril(diagonal=past)
-            out = torch.nn.functional.scaled_dot_product_attention(qs, ks, vs, attn_mask=mask)
+            out = torch.nn.functional.scaled_dot_product_attention(qs, ks, vs, attn_mask=mask, enable_gqa=gqa)
         out = out.transpose(1, 2).reshape(b, t, self.hidden_size).contiguous()
-        s, z, q = self._token_quant(out) if self.activation == "token" else self.attn_quantizer2(out)
-        return self.o_proj(q, s, z, x_is_packed=True), cache
+        if (self.activation == "token" and self.fused and self.record is None and b * t <= 2
+                and self.hidden_size == 4096):
+            # decode: the quantiser runs inside the GEMM's own launch (same bits as the two launches)
+            return self.o_proj.forward_online(out, hadamard="exact"), cache
+        s, z, q = self._token_quant("attn_out", out) if self.activation == "token" else self._group_quant("attn_out", self.attn_quantizer2, out)
+        y = self.o_proj(q, s, z, x_is_packed=True)
+        self._tap("o_proj", y)
+        return y, cache
+
+    def _group_quant(self, stage, quantizer, x):
+        s, z, q = quantizer(x)
+        self._tap(stage + ".input", x.reshape(-1, x.size(-1)))
+        self._tap(stage + ".codes", q.reshape(-1, q.size(-1)))
+        self._tap(stage + ".scales", s.reshape(-1, s.size(-1)))
+        return s, z, q
 
     def mlp(self, x):
-        s, z, q = self._norm_quant(self.post_attention_layernorm, self.mlp_quantizer1, x)
+        s, z, q = self._norm_quant("mlp_in", self.post_attention_layernorm, "post_attention_layernorm",
+                                   self.mlp_quantizer1, x)
         gate, up = self._project([self.gate_proj, self.up_proj], q, s, z)
+        self._tap("gate_proj", gate), self._tap("up_proj", up)
         if self.activation == "token":
-            s, z, q = self._token_quant(torch.nn.functional.silu(gate) * up)
-        elif self.fused:
+            s, z, q = self._token_quant("mlp_mid", torch.nn.functional.silu(gate) * up)
+        elif self.fused and self.record is None:
             s, z, q = self._silu_mul_quant(gate, up)
         else:
-            s, z, q = self.mlp_quantizer2(torch.nn.functional.silu(gate) * up)
-        return self.down_proj(q, s, z, x_is_packed=True)
+            s, z, q = self._group_quant("mlp_mid", self.mlp_quantizer2, torch.nn.functional.silu(gate) * up)
+        y = self.down_proj(q, s, z, x_is_packed=True)
+        self._tap("down_proj", y)
+        return y
 
-    def forward(self, x, cos, sin, kv_cache=None):
-        attn, cache = self.attention(x, cos, sin, kv_cache)
+    def forward(self, x, cos, sin, kv_cache=None, positions=None):
+        attn, cache = self.attention(x, cos, sin, kv_cache, positions)
         x = x + attn
         return x + self.mlp(x), cache
 

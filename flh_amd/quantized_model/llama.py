@@ -1,0 +1,122 @@
+"""A W4A4 Llama model around the decoder layer: embedding, N layers, final norm, fp16 language-model head, and a
+decode step that runs from a preallocated key / value cache and can be captured into one graph.
+
+Data flow of the reference's FLH_LlamaForCausalLM.forward (flh/quantized_model/modeling_llama.py:668-693:
+embedding -> [group configuration only: Hadamard of every 128 channels of the embeddings] -> decoder layers ->
+final RMSNorm -> lm_head), with the layers of decoder_layer.py.  The int4 linears are this library's kernels; the
+embedding, RoPE, attention, norms outside the fused launches and the head are stock torch ops, as in the reference.
+Weights are random (there are no checkpoints here): `random_init` draws fp16 weights layer by layer on the device and
+quantises them through the same kernels a loader would use.
+"""
+import math
+
+import torch
+
+from ..nn.normalization import RMSNorm
+from ..nn.quantization import fast_hadamard_transform
+from .decoder_layer import StaticKVCache, W4A4DecoderLayer, rotary_tables
+
+
+class LlamaShape:
+    """The numbers that define a Llama-style stack."""
+
+    def __init__(self, hidden_size=4096, num_heads=32, num_kv_heads=8, intermediate_size=14336, num_layers=32,
+                 vocab_size=128256, eps=1e-5, rope_theta=500000.0):
+        self.hidden_size, self.num_heads, self.num_kv_heads = hidden_size, num_heads, num_kv_heads
+        self.intermediate_size, self.num_layers, self.vocab_size = intermediate_size, num_layers, vocab_size
+        self.eps, self.rope_theta = eps, rope_theta
+        self.head_dim = hidden_size // num_heads
+
+    @classmethod
+    def llama3_8b(cls, num_layers=32):
+        return cls(4096, 32, 8, 14336, num_layers, 128256, 1e-5, 500000.0)
+
+    @classmethod
+    def llama2_7b(cls, num_layers=32):
+        return cls(4096, 32, 32, 11008, num_layers, 32000, 1e-5, 10000.0)
+
+
+class W4A4LlamaModel(torch.nn.Module):
+    def __init__(self, shape, activation="token", weight_group_size=128, fused=True, device="cpu"):
+        super().__init__()
+        self.shape, self.activation = shape, activation
+        self.embed_tokens = torch.nn.Embedding(shape.vocab_size, shape.hidden_size, device=device, dtype=torch.float16)
+        self.layers = torch.nn.ModuleList(
+            W4A4DecoderLayer(shape.hidden_size, shape.num_heads, shape.num_kv_heads, shape.intermediate_size, shape.eps,
+                             128, weight_group_size, fused, device, activation) for _ in range(shape.num_layers))
+        self.norm = RMSNorm(shape.hidden_size, shape.eps).to(device)
+        self.lm_head = torch.nn.Linear(shape.hidden_size, shape.vocab_size, bias=False, device=device, dtype=torch.float16)
+
+    @classmethod
+    def random_init(cls, shape, activation="token", weight_group_size=128, fused=True, device="cuda", seed=0):
+        """Random fp16 weights ~ N(0, 1/K) per linear (norm weights ~ U(0.5, 1.5)), quantised on the device one layer
+        at a time so that no more than one layer's fp16 weights exist at once."""
+        model = cls(shape, activation, weight_group_size, fused, device="meta")
+        model.embed_tokens = torch.nn.Embedding(shape.vocab_size, shape.hidden_size, device=device, dtype=torch.float16)
+        model.lm_head = torch.nn.Linear(shape.hidden_size, shape.vocab_size, bias=False, device=device, dtype=torch.float16)
+        model.norm = RMSNorm(shape.hidden_size, shape.eps).to(device)
+        gen = torch.Generator(device=device).manual_seed(seed)
+        with torch.no_grad():
+            model.embed_tokens.weight.normal_(0.0, 1.0, generator=gen)
+            model.lm_head.weight.normal_(0.0, 1.0 / math.sqrt(shape.hidden_size), generator=gen)
+            model.norm.weight.uniform_(0.5, 1.5, generator=gen)
+            kv = shape.num_kv_heads * shape.head_dim
+            dims = {"q_proj": (shape.hidden_size, shape.hidden_size), "k_proj": (kv, shape.hidden_size),
+                    "v_proj": (kv, shape.hidden_size), "o_proj": (shape.hidden_size, shape.hidden_size),
+                    "gate_proj": (shape.intermediate_size, shape.hidden_size),
+                    "up_proj": (shape.intermediate_size, shape.hidden_size),
+                    "down_proj": (shape.hidden_size, shape.intermediate_size)}
+            layers = []
+            for _ in range(shape.num_layers):
+                w = {name: (torch.randn(n, k, device=device, generator=gen) / math.sqrt(k)).half() for name, (n, k) in dims.items()}
+                for name in ("input_layernorm", "post_attention_layernorm"):
+                    w[name] = (torch.rand(shape.hidden_size, device=device, generator=gen) + 0.5).half()
+                layers.append(W4A4DecoderLayer.from_float(w, shape.num_heads, shape.num_kv_heads, shape.eps, 128,
+                                                          weight_group_size if activation == "token" else 128, fused,
+                                                          activation))
+                del w
+            model.layers = torch.nn.ModuleList(layers)
+        return model
+
+    def new_cache(self, batch, max_len):
+        s = self.shape
+        dev = self.embed_tokens.weight.device
+        return StaticKVCache(s.num_layers, batch, s.num_kv_heads, max_len, s.head_dim, dev)
+
+    def embed(self, input_ids):
+        x = self.embed_tokens(input_ids)
+        if self.activation == "group":     # modeling_llama.py:672: the rotations of this arrangement live in the weights
+            x = fast_hadamard_transform(x, group_size=128, normalize=True)
+        return x
+
+    def forward(self, input_ids, positions, cache=None, return_hidden=False):
+        """input_ids [B, T] int64, positions [T] int64 (the same for every sequence of the batch).  cache: None (a
+        fresh prefill without cache), or a StaticKVCache whose kv_len the caller has set to the number of slots
+        attention may read (>= positions.max() + 1).  Returns logits [B, T, vocab] fp16 (or the final hidden state)."""
+        x = self.embed(input_ids)
+        cos, sin = rotary_tables(positions, self.shape.head_dim, self.shape.rope_theta)
+        for i, layer in enumerate(self.layers):
+            x, _ = layer(x, cos, sin, cache.layer(i) if cache is not None else None, positions)
+        x = self.norm(x)
+        return x if return_hidden else self.lm_head(x)
+
+    def capture_decode_step(self, batch, kv_len, cache=None, with_head=True):
+        """Record one decode step (batch x 1 token, attention over `kv_len` cached positions, the new token in slot
+        kv_len - 1) into a graph.  Returns (graph, static): `static` holds the input ids, the position tensor and the
+        output logits the replays read and write; the cache must already hold the earlier positions."""
+        dev = self.embed_tokens.weight.device
+        cache = cache if cache is not None else self.new_cache(batch, kv_len)
+        cache.kv_len = kv_len
+        ids = torch.zeros(batch, 1, dtype=torch.int64, device=dev)
+        pos = torch.full((1,), kv_len - 1, dtype=torch.int64, device=dev)
+        side = torch.cuda.Stream(device=dev)
+        side.wait_stream(torch.cuda.current_stream(dev))
+        with torch.cuda.stream(side), torch.no_grad():
+            for _ in range(2):              # every kernel variant runs once eagerly before the capture
+                out = self.forward(ids, pos, cache, return_hidden=not with_head)
+        torch.cuda.current_stream(dev).wait_stream(side)
+        torch.cuda.synchronize(dev)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph), torch.no_grad():
+            out = self.forward(ids, pos, cache, return_hidden=not with_head)
+        return graph, {"input_ids": ids, "positions": pos, "output": out, "cache": cache}

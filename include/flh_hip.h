@@ -87,13 +87,11 @@ int flh_rotate_quant_gemm_i4_o16_multi(const flh_half* x, int count, const uint8
                                        const flh_half* const* b_scale, flh_half* const* D, const size_t* N, size_t M,
                                        size_t K, int b_cols, void* stream);
 
-/* Diagnostic (no counterpart in the reference; nothing in the product path calls it): one launch of a loop of nothing
- * but the int8 matrix instruction -- 512 workgroups x 4 waves x iters x 16 instructions of 65536 integer operations
- * each -- on operands of a chosen kind: pattern 0 zeros, 1 int4 codes x 16 (what the GEMM feeds its matrix pipes),
- * 2 random bytes, 3 codes + 8 (bytes 0..15) in both operands, 4 codes + 8 in the first and codes x 16 in the second
- * operand, 5 sign-extended codes (bytes -8..7).  The caller times it.  The sustained clock of the part depends on the operand values, so this is
- * the ceiling a GEMM on such operands can be compared with beside the published peak. */
-int flh_probe_mfma_i8(int pattern, int iters, void* stream);
+/* Test and tuning hook (no counterpart in the reference): overrides, process-wide, the tile (64, 128 or 256 rows;
+ * 0 = automatic) and the split of K inside a workgroup (1, 2 or 4; 0 = automatic) that flh_gemm_i4_o16 and
+ * flh_gemm_f6_o16 would choose from the shape.  Every variant gives the same bits; the tests use this to reach
+ * all of them.  Combinations a kernel does not offer fall back to the nearest one it does. */
+int flh_gemm_set_tuning(int tile, int k_split);
 
 /* The raw int32 accumulators C[m,n] = sum_k A[m,k] * B[n,k] (for parity checks of the
  * contraction itself; the reference keeps them in registers,

@@ -53,9 +53,9 @@ def test_gemm_f6_int32_bit_exact(ops, m, n, k):
 
 @pytest.mark.parametrize("tile", [256, 128, 64])
 @pytest.mark.parametrize("k", [1536, 1408, 128])      # even / odd number of K steps, a single step
-def test_gemm_f6_every_tile(ops, tile, k, monkeypatch):
+def test_gemm_f6_every_tile(ops, tile, k, gemm_tuning):
     from oracle import gemm as G
-    monkeypatch.setenv("FLH_GEMM_TILE", str(tile))
+    gemm_tuning(tile)
     m, n = 300, 264
     rng = np.random.default_rng(tile + k)
     a = rng.integers(-8, 8, size=(m, k), dtype=np.int8)

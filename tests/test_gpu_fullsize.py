@@ -103,6 +103,31 @@ def test_decode_full_matrices_bit_exact(ops, m, n, k):
         assert np.array_equal(d.view(np.uint16), ref.view(np.uint16))
 
 
+@pytest.mark.parametrize("m", [8, 256])
+@pytest.mark.parametrize("n,k", sorted(set(LLAMA2 + LLAMA3)))
+def test_batch_8_and_256_full_width(ops, m, n, k):
+    """M = 8 (decode batch of the Llama-3 step) and M = 256 (the short prefill, which selects the 64 x 64 tile with K
+    split over four wave quads) at the full Llama widths: whole int32 matrices against the oracle, the one-scale-per-row
+    epilogue bit for bit, the group epilogue (one scale per token, weight groups of 128) bit-equal to the FMA oracle."""
+    from oracle import gemm as G
+    a, b = codes(m, k, 11 * m + n), codes(n, k, 13 * m + k)
+    ap, bp = syn.pack_codes(a), syn.pack_codes(b)
+    print(f"case full-width m={m} n={n} k={k}", flush=True)
+    acc = G.int_gemm(a, b)
+    assert np.array_equal(host(ops.gemm_i4_int32(dev(ap), dev(bp))), acc)
+    rng = np.random.default_rng(n + m + k)
+    sa = rng.uniform(0.01, 0.5, size=(m, 1)).astype(np.float16)
+    sb = syn.weight_scales(n, 1, seed=k)
+    d = host(ops.gemm_i4_dequant_o16(dev(ap), dev(bp), dev(sa), dev(sb)))
+    ref, _ = G.gemm_i4_dequant(ap, bp, sa, sb)
+    assert np.array_equal(d.view(np.uint16), ref.view(np.uint16))
+    sbg = syn.weight_scales(n, k // 128, seed=k + 1)
+    d = host(ops.gemm_i4_dequant_o16(dev(ap), dev(bp), dev(sa), dev(sbg)))
+    ref, _ = G.gemm_i4_dequant(ap, bp, sa, sbg)
+    assert np.allclose(d.astype(np.float64), ref.astype(np.float64), rtol=1e-3, atol=1e-2)
+    assert np.array_equal(d.view(np.uint16), ref.view(np.uint16))
+
+
 def test_rotate_quant_exact_mode_whole_batch(ops):
     """M = 2048, K = 4096: every row against the float32-butterfly oracle, bit for bit."""
     from oracle import linear as L

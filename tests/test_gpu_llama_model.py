@@ -1,0 +1,269 @@
+"""The W4A4 Llama harness (flh_amd.quantized_model) against the CPU oracle layer (oracle/layer.py), at full width.
+
+Two workloads:
+  * the Llama-3-8B decode step: batch {1, 8, 16} x 1 token, attention over 2048 cached positions, grouped queries
+    32 / 8, intermediate 14336 with the 28 x 512 online rotation, group-of-128 weight scales, per-token activation
+    scales, final norm and the fp16 head of 128 256 rows -- two full-width layers here (the 32 of the full model repeat
+    them; bench.py runs all 32);
+  * a Llama-2-7B decoder layer at 8 x 512 tokens (per-token activations, per-channel weight scales, 172 x 64 rotation).
+
+Every stage of the device layer is checked with the oracle fed the device's own input of that stage (its `record`
+taps): quantised operands bit for bit where the arithmetic is this library's (the float32-butterfly rotation of 4096
+and the quantiser), by mismatch rate where the device's float32 order is not the oracle's (RMSNorm statistics in front
+of the rotation; the matrix-core rotation of 11008 / 14336); every linear's fp16 output within rtol 1e-3 / atol 1e-2 of
+the oracle GEMM on the same codes and scales; the attention block (RoPE, cache write, grouped queries, masking) against
+the float64 attention.  On top, the free-running oracle model from the same inputs bounds the end-to-end difference.
+"""
+import numpy as np
+import pytest
+import torch
+
+from flh_amd.quantized_model import LlamaShape, StaticKVCache, W4A4DecoderLayer, W4A4LlamaModel, rotary_tables
+
+pytestmark = pytest.mark.gpu
+
+
+def host(t):
+    return t.detach().cpu().numpy()
+
+
+def oracle_weights(layer, activation, weight_group):
+    from oracle import layer as OL
+    packed = {n: host(getattr(layer, n).w_packed).reshape(getattr(layer, n).out_features, -1) for n in layer.PROJECTIONS}
+    scales = {n: host(getattr(layer, n).w_scale).reshape(getattr(layer, n).out_features, -1) for n in layer.PROJECTIONS}
+    norms = {n: host(getattr(layer, n).weight).astype(np.float16) for n in ("input_layernorm", "post_attention_layernorm")}
+    for n in norms:      # the device holds float32 norm weights that came from fp16 values: the conversion is exact
+        assert np.array_equal(norms[n].astype(np.float32), host(getattr(layer, n).weight))
+    return OL.LayerWeights(packed, scales, norms, layer.num_heads, layer.num_kv_heads, layer.eps, activation, weight_group)
+
+
+def mismatch(a, b):
+    return float(np.mean(a != b))
+
+
+def nibble_step(a, b):
+    """largest difference between the int4 codes of two packed arrays"""
+    from oracle.pack import unpack_i4
+    return int(np.abs(unpack_i4(a).astype(np.int32) - unpack_i4(b).astype(np.int32)).max())
+
+
+def ulp_distance(a, b):
+    return int(np.abs(a.view(np.int16).astype(np.int32) - b.view(np.int16).astype(np.int32)).max())
+
+
+def check_layer_stages(rec, w, x_rows, cos, sin, b, t, past_kv, sample=None, label=""):
+    """rec: the device layer's taps (host arrays); w: oracle weights; x_rows fp16 [b * t, hidden]: the layer's input;
+    past_kv: None or (keys, values) host arrays [b, Hkv, past, d].  `sample`: row indices for the GEMM checks."""
+    from oracle import gemm as G
+    from oracle import layer as OL
+    from oracle import prologue
+    rows = np.arange(b * t) if sample is None else sample
+    hidden = x_rows.shape[1]
+    hd = hidden // w.num_heads
+
+    def gemm_stage(name, codes, scales):
+        ref, _ = G.gemm_i4_dequant(codes[rows], w.packed[name], scales[rows], w.scales[name], group=w.weight_group)
+        got = rec[name][rows]
+        assert np.allclose(got.astype(np.float64), ref.astype(np.float64), rtol=1e-3, atol=1e-2), (label, name)
+        return mismatch(got.view(np.uint16), ref.view(np.uint16))
+
+    report = {}
+    # quantiser behind RMSNorm: the device's float32 statistics / rsqrt are its own -> codes by mismatch rate
+    assert np.array_equal(rec["attn_in.input"], x_rows)
+    q, s, _ = OL.quantise(w, x_rows, w.norms["input_layernorm"])
+    report["attn_in codes"] = mismatch(rec["attn_in.codes"], q)
+    assert report["attn_in codes"] < 2e-3 and nibble_step(rec["attn_in.codes"], q) <= 1, (label, report)
+    assert ulp_distance(rec["attn_in.scales"], s) <= 2
+    for name in ("q_proj", "k_proj", "v_proj"):
+        report[name] = gemm_stage(name, rec["attn_in.codes"], rec["attn_in.scales"])
+    # attention block from the device's own projections
+    heads = {n: rec[n].reshape(b, t, nh, hd).transpose(0, 2, 1, 3) for n, nh in
+             (("q_proj", w.num_heads), ("k_proj", w.num_kv_heads), ("v_proj", w.num_kv_heads))}
+    qs, ks, vs = OL.apply_rotary(heads["q_proj"], cos, sin), OL.apply_rotary(heads["k_proj"], cos, sin), heads["v_proj"]
+    past = 0
+    if past_kv is not None:
+        past = past_kv[0].shape[2]
+        ks, vs = np.concatenate((past_kv[0], ks), axis=2), np.concatenate((past_kv[1], vs), axis=2)
+    att = OL.attention_f64(qs, ks, vs, past).transpose(0, 2, 1, 3).reshape(b * t, hidden)
+    diff = np.abs(rec["attn_out.input"].astype(np.float64) - att.astype(np.float64))
+    report["attention max abs diff"] = float(diff.max())
+    assert diff.max() <= 4e-3 * max(1.0, float(np.abs(att.astype(np.float64)).max())), (label, report)
+    # quantiser without norm at the hidden width: this library's arithmetic end to end -> bit for bit
+    q, s, _ = OL.quantise(w, rec["attn_out.input"])
+    if w.activation == "group" or hidden & (hidden - 1) == 0:
+        assert np.array_equal(rec["attn_out.codes"], q) and np.array_equal(rec["attn_out.scales"].view(np.uint16), s.view(np.uint16)), label
+    report["o_proj"] = gemm_stage("o_proj", rec["attn_out.codes"], rec["attn_out.scales"])
+    resid = (x_rows.astype(np.float32) + rec["o_proj"].astype(np.float32)).astype(np.float16)
+    assert np.array_equal(rec["mlp_in.input"], resid), label
+    q, s, _ = OL.quantise(w, resid, w.norms["post_attention_layernorm"])
+    report["mlp_in codes"] = mismatch(rec["mlp_in.codes"], q)
+    assert report["mlp_in codes"] < 2e-3 and nibble_step(rec["mlp_in.codes"], q) <= 1, (label, report)
+    for name in ("gate_proj", "up_proj"):
+        report[name] = gemm_stage(name, rec["mlp_in.codes"], rec["mlp_in.scales"])
+    mid = prologue.silu_mul_f16(rec["gate_proj"], rec["up_proj"])
+    report["silu*up fp16 mismatch"] = mismatch(rec["mlp_mid.input"].view(np.uint16), mid.view(np.uint16))
+    assert report["silu*up fp16 mismatch"] < 5e-3, (label, report)          # device exp / division: last-bit differences
+    # the intermediate width (172 x 64 / 28 x 512): matrix-core rotation on the device, float32 matmul_hadU in the oracle
+    q, s, _ = OL.quantise(w, rec["mlp_mid.input"])
+    report["mlp_mid codes"] = mismatch(rec["mlp_mid.codes"], q)
+    inter = rec["mlp_mid.input"].shape[1]
+    if w.activation == "token" and inter & (inter - 1):
+        assert report["mlp_mid codes"] < 3e-3 and nibble_step(rec["mlp_mid.codes"], q) <= 1, (label, report)
+        assert ulp_distance(rec["mlp_mid.scales"], s) <= 2
+    else:
+        assert np.array_equal(rec["mlp_mid.codes"], q) and np.array_equal(rec["mlp_mid.scales"].view(np.uint16), s.view(np.uint16)), label
+    report["down_proj"] = gemm_stage("down_proj", rec["mlp_mid.codes"], rec["mlp_mid.scales"])
+    out = (resid.astype(np.float32) + rec["down_proj"].astype(np.float32)).astype(np.float16)
+    return out, report
+
+
+@pytest.fixture(scope="module")
+def llama3_two_layers():
+    assert torch.cuda.is_available()
+    shape = LlamaShape.llama3_8b(num_layers=2)
+    with torch.no_grad():
+        model = W4A4LlamaModel.random_init(shape, activation="token", weight_group_size=128, fused=True, seed=3)
+    weights = [oracle_weights(l, "token", 128) for l in model.layers]
+    return model, weights
+
+
+@pytest.mark.parametrize("batch", [1, 8, 16])
+def test_llama3_decode_step_against_the_oracle(llama3_two_layers, batch):
+    from oracle import layer as OL
+    model, weights = llama3_two_layers
+    shape = model.shape
+    kv_len = 2048
+    gen = torch.Generator(device="cuda").manual_seed(100 + batch)
+    cache = model.new_cache(batch, kv_len)
+    for i in range(shape.num_layers):       # a cache state as a 2047-token prefill would leave it: random keys / values
+        cache.keys[i][:, :, :kv_len - 1].normal_(0.0, 1.0, generator=gen)
+        cache.values[i][:, :, :kv_len - 1].normal_(0.0, 1.0, generator=gen)
+    past = [(host(cache.keys[i][:, :, :kv_len - 1]), host(cache.values[i][:, :, :kv_len - 1])) for i in range(shape.num_layers)]
+    cache.kv_len = kv_len
+    ids = torch.randint(0, shape.vocab_size, (batch, 1), device="cuda", generator=gen)
+    pos = torch.tensor([kv_len - 1], device="cuda")
+    print(f"case llama3 decode step batch={batch}", flush=True)
+    # recorded run (module-by-module o_proj so that every stage is visible)
+    recs = [dict() for _ in model.layers]
+    for layer, r in zip(model.layers, recs):
+        layer.record = r
+    with torch.no_grad():
+        hidden_rec = model(ids, pos, cache, return_hidden=True)
+    for layer in model.layers:
+        layer.record = None
+    new_k = [host(cache.keys[i][:, :, kv_len - 1]) for i in range(shape.num_layers)]
+    # the production run: fused decode path, then head
+    with torch.no_grad():
+        logits = model(ids, pos, cache)
+        hidden = model(ids, pos, cache, return_hidden=True)
+    assert torch.equal(hidden, hidden_rec), "the single-launch decode path must give the recorded path's bits"
+    for i in range(shape.num_layers):       # replaying the step rewrites the same slot with the same keys
+        assert np.array_equal(host(cache.keys[i][:, :, kv_len - 1]), new_k[i])
+        assert np.array_equal(host(cache.keys[i][:, :, :kv_len - 1]), past[i][0])
+
+    x = host(model.embed(ids)).reshape(batch, shape.hidden_size)
+    cos, sin = OL.rotary_tables(np.array([kv_len - 1]), shape.head_dim, shape.rope_theta)
+    dcos, dsin = rotary_tables(pos, shape.head_dim, shape.rope_theta)
+    assert np.abs(host(dcos).astype(np.float64) - cos.astype(np.float64)).max() <= 1e-3
+    assert np.abs(host(dsin).astype(np.float64) - sin.astype(np.float64)).max() <= 1e-3
+    cos, sin = host(dcos), host(dsin)           # the device's tables (they differ from float64 in the last fp16 bit at most)
+    rows = x
+    for i, (w, r) in enumerate(zip(weights, recs)):
+        rec = {k: host(v) for k, v in r.items()}
+        rows, report = check_layer_stages(rec, w, rows, cos, sin, batch, 1, past[i], label=f"layer {i} batch {batch}")
+        print(f"  layer {i}: " + ", ".join(f"{k} {v:.2e}" for k, v in report.items()), flush=True)
+    # final norm and head (stock torch ops) on the device's last hidden state
+    from oracle import prologue
+    fn = host(model.norm.weight).astype(np.float16)
+    want_hidden = prologue.rmsnorm_f16(rows, fn, shape.eps)
+    got_hidden = host(hidden).reshape(batch, -1)
+    assert mismatch(got_hidden.view(np.uint16), want_hidden.view(np.uint16)) < 5e-3
+    assert np.allclose(got_hidden.astype(np.float64), want_hidden.astype(np.float64), rtol=2e-3, atol=1e-3)
+    sample = np.random.default_rng(batch).choice(shape.vocab_size, 2048, replace=False)
+    head = host(model.lm_head.weight[torch.from_numpy(sample).cuda()]).astype(np.float64)
+    want_logits = got_hidden.astype(np.float64) @ head.T
+    got_logits = host(logits).reshape(batch, -1)[:, sample].astype(np.float64)
+    assert logits.shape == (batch, 1, shape.vocab_size)
+    assert np.allclose(got_logits, want_logits, rtol=2e-3, atol=2e-2)
+    # free-running oracle model from the same inputs: bounds what the stage-wise differences add up to
+    free, _ = OL.model_step(weights, x.reshape(batch, 1, -1), np.array([kv_len - 1]), shape.head_dim, shape.rope_theta,
+                            caches=past, final_norm=fn, eps=shape.eps)
+    err = np.linalg.norm(free.reshape(batch, -1).astype(np.float64) - got_hidden.astype(np.float64)) / np.linalg.norm(got_hidden.astype(np.float64))
+    print(f"  free-running oracle vs device, final hidden state: relative difference {err:.3e}", flush=True)
+    assert err < 0.05
+
+
+def test_llama3_decode_step_replays_from_a_graph(llama3_two_layers):
+    """The whole step (two layers, norm, head) captured once and replayed: the same logits as the eager step, on
+    every replay, also after the token and the cache contents change between replays."""
+    model, _ = llama3_two_layers
+    shape = model.shape
+    batch, kv_len = 8, 2048
+    gen = torch.Generator(device="cuda").manual_seed(5)
+    graph, st = model.capture_decode_step(batch, kv_len)
+    cache = st["cache"]
+    for round_ in range(3):
+        for i in range(shape.num_layers):
+            cache.keys[i][:, :, :kv_len - 1].normal_(0.0, 1.0, generator=gen)
+            cache.values[i][:, :, :kv_len - 1].normal_(0.0, 1.0, generator=gen)
+        st["input_ids"].copy_(torch.randint(0, shape.vocab_size, (batch, 1), device="cuda", generator=gen))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        got = st["output"].clone()
+        with torch.no_grad():
+            want = model(st["input_ids"], st["positions"], cache)
+        torch.cuda.synchronize()
+        assert torch.equal(got, want), f"replay {round_}"
+
+
+def test_llama2_layer_8x512_against_the_oracle():
+    """BASELINE configuration 4: one Llama-2-7B decoder layer, batch 8 x 512 tokens, per-token activations with the
+    whole-row online rotation (4096, and 172 x 64 in front of down_proj), per-channel weight scales.  Quantiser and
+    attention stages on the whole batch, GEMM stages on 192 sampled tokens (the oracle's matrix products)."""
+    from oracle import layer as OL
+    b, t, hidden, heads, inter = 8, 512, 4096, 32, 11008
+    gen = torch.Generator(device="cuda").manual_seed(21)
+    dims = {"q_proj": (hidden, hidden), "k_proj": (hidden, hidden), "v_proj": (hidden, hidden), "o_proj": (hidden, hidden),
+            "gate_proj": (inter, hidden), "up_proj": (inter, hidden), "down_proj": (hidden, inter)}
+    w16 = {n: (torch.randn(s, device="cuda", generator=gen) / s[1] ** 0.5).half() for n, s in dims.items()}
+    for n in ("input_layernorm", "post_attention_layernorm"):
+        w16[n] = (torch.rand(hidden, device="cuda", generator=gen) + 0.5).half()
+    with torch.no_grad():
+        layer = W4A4DecoderLayer.from_float(w16, heads, heads, activation="token", fused=True)
+    del w16
+    w = oracle_weights(layer, "token", 128)
+    assert w.scales["q_proj"].shape == (hidden, 1)
+    x = torch.randn(b, t, hidden, device="cuda", generator=gen).half()
+    x[..., ::97] *= 12.0                                 # outlier channels
+    cos, sin = rotary_tables(torch.arange(t, device="cuda"), hidden // heads)
+    print("case llama2 layer 8x512", flush=True)
+    rec = {}
+    layer.record = rec
+    with torch.no_grad():
+        y_rec, (k_rec, v_rec) = layer(x, cos, sin)
+    layer.record = None
+    with torch.no_grad():
+        y, (k, v) = layer(x, cos, sin)
+    assert torch.equal(y, y_rec) and torch.equal(k, k_rec) and torch.equal(v, v_rec)
+    rec = {kk: host(vv) for kk, vv in rec.items()}
+    sample = np.sort(np.random.default_rng(4).choice(b * t, 192, replace=False))
+    out, report = check_layer_stages(rec, w, host(x).reshape(b * t, hidden), host(cos), host(sin), b, t, None,
+                                     sample=sample, label="llama2 8x512")
+    print("  " + ", ".join(f"{kk} {vv:.2e}" for kk, vv in report.items()), flush=True)
+    assert np.array_equal(host(y).reshape(b * t, hidden), out)
+    # whole-batch invariants of the outputs the sampled GEMM checks did not see: every row of every projection is
+    # the row the same launch gives for that token alone (prefill kernel against the decode kernel, same bits)
+    ops = __import__("flh_amd")._CUDA
+    for name, codes, scales in (("q_proj", "attn_in", "attn_in"), ("down_proj", "mlp_mid", "mlp_mid")):
+        lin = getattr(layer, name)
+        pick = torch.from_numpy(sample[:48]).cuda()
+        qd, sd = torch.from_numpy(rec[codes + ".codes"]).cuda()[pick].contiguous(), torch.from_numpy(rec[scales + ".scales"]).cuda()[pick].contiguous()
+        small = ops.gemm_i4_dequant(qd, lin.w_packed.view(lin.out_features, -1), sd, lin.w_scale, 128)
+        assert np.array_equal(host(small), rec[name][sample[:48]])
+    # free-running oracle on a few sequences would repeat the stage checks; the end-to-end bound on one sequence:
+    free, _ = OL.decoder_layer(w, host(x[:1]), host(cos), host(sin))
+    got = host(y[:1]).astype(np.float64)
+    err = np.linalg.norm(free.astype(np.float64) - got) / np.linalg.norm(got - host(x[:1]).astype(np.float64))
+    print(f"  free-running oracle layer vs device (sequence 0): relative difference of the update {err:.3e}", flush=True)
+    assert err < 0.05

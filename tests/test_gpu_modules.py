@@ -300,3 +300,34 @@ def test_forward_many_on_the_six_bit_path(group):
     assert all(layer._w6 is not None for layer in layers)
     for a, b in zip(got, want):
         assert torch.equal(a, b)
+
+
+@pytest.mark.parametrize("g", [128, 64])
+def test_hql_linear4bit_alias(g):
+    """The legacy names of the reference's linear benchmark (benchmark_linear4bit.py:495-508): weights prepared with
+    hql.had_and_quant, forward on fp16 activations.  Codes / scales of both operands against the oracle's group kernel,
+    the output against the oracle GEMM on them, and against x @ W.T as the benchmark's own error check does."""
+    from oracle import gemm as G
+    from oracle import quant as Q
+    from oracle.pack import pack_i4
+    import flh_amd.hql as hql
+    hql.install_as_hql()
+    from hql.nn import Linear4bit
+    k, n, m = 1024, 384, 40
+    rng = np.random.default_rng(g)
+    w = (rng.standard_normal((n, k)) * 0.02).astype(np.float16)
+    x = syn.activations(m, k, seed=3 + g)
+    layer = Linear4bit(k, n, bias=False, dtype=torch.float16, group_size=g).cuda()
+    qw, sw = hql.had_and_quant(dev(w).view(-1, g))
+    layer.weight.copy_(qw.reshape(-1, k // 2))
+    layer.weight_scales.copy_(sw.reshape(-1, k // g))
+    qwr, swr, _ = Q.kernel_had_and_quant(w.reshape(-1, g), g, True)
+    assert np.array_equal(host(layer.weight), pack_i4(qwr).reshape(n, k // 2))
+    assert np.array_equal(host(layer.weight_scales).view(np.uint16), swr.reshape(n, -1).view(np.uint16))
+    y = host(layer(dev(x)))
+    qxr, sxr, _ = Q.kernel_had_and_quant(x.reshape(-1, g), g, True)
+    sx = (sxr.astype(np.float32) * np.float32(1.0 / g)).astype(np.float16).reshape(m, -1)
+    ref, _ = G.gemm_i4_dequant(pack_i4(qxr).reshape(m, k // 2), pack_i4(qwr).reshape(n, k // 2), sx, swr.reshape(n, -1), group=g)
+    assert np.allclose(y.astype(np.float64), ref.astype(np.float64), rtol=1e-3, atol=1e-2)
+    full = x.astype(np.float64) @ w.astype(np.float64).T
+    assert np.linalg.norm(y - full) / np.linalg.norm(full) < 0.3

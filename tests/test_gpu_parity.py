@@ -50,12 +50,11 @@ def test_gemm_int32_bit_exact(ops, m, n, k):
 
 @pytest.mark.parametrize("tile,ks", [(256, 1), (256, 2), (128, 1), (128, 2), (64, 1), (64, 2), (64, 4)])
 @pytest.mark.parametrize("k", [1536, 1408])     # 12 resp. 11 K steps: even and uneven splits
-def test_gemm_every_tile_and_k_split(ops, tile, ks, k, monkeypatch):
+def test_gemm_every_tile_and_k_split(ops, tile, ks, k, gemm_tuning):
     """The tuning overrides select each tile shape and in-workgroup K split directly; all of them
     must give the same exact integers and the same bit-exact fp16 outputs."""
     from oracle import gemm as G
-    monkeypatch.setenv("FLH_GEMM_TILE", str(tile))
-    monkeypatch.setenv("FLH_GEMM_KS", str(ks))
+    gemm_tuning(tile, ks)
     m, n = 300, 264
     rng = np.random.default_rng(tile + ks + k)
     a = rng.integers(-8, 8, size=(m, k), dtype=np.int8)

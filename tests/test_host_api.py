@@ -27,6 +27,13 @@ def test_library_exports_every_declared_symbol():
     lib = _lib.load()          # raises if the .so is missing or a symbol is not exported
     assert lib.flh_abi_version() == 1
     assert lib.flh_last_error() == b""
+    # the reference's C++-linkage functions: one mangled export per declaration of the second header
+    native = (ROOT / "include" / "flh_reference_native.h").read_text()
+    declared_cxx = set(re.findall(r"^void\s+(\w+)\(", native, re.M))
+    assert declared_cxx == set(_lib._SIG_CXX), declared_cxx ^ set(_lib._SIG_CXX)
+    for name, mangled in _lib._SIG_CXX.items():
+        assert name in mangled and "6__half" in mangled
+        assert getattr(lib, mangled) is not None
 
 
 def test_argument_errors_come_back_before_any_launch():
