@@ -100,6 +100,8 @@ def main():
     ap.add_argument("--cpu-sample-tokens", type=int, default=2048)
     ap.add_argument("--no-vendor-reference", action="store_true",
                     help="skip timing the vendor library's int8 / fp16 GEMM on the same shapes")
+    ap.add_argument("--no-decode-model", action="store_true",
+                    help="skip the 32-layer Llama-3-8B decode step (about 6 GB of random weights)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also launch three elementwise passes over 256 MiB (read 256 MiB, write 256 MiB): the "
                          "known-size kernel that hardware-counter readings (FETCH_SIZE / WRITE_SIZE) are scaled by")
@@ -232,15 +234,6 @@ def main():
             pairs.append((e0, e1))
         torch.cuda.synchronize()
         return float(np.median([a.elapsed_time(b) * 1e3 for a, b in pairs]))
-
-    # what the matrix pipes sustain on nothing but the int8 matrix instruction, by operand values (the part's clock
-    # follows the switching activity): the GEMM's practical ceiling is the rate on operands like its own
-    def matrix_rate(pattern, iters=4000):
-        ops.probe_mfma_i8(pattern, iters)
-        us = timed([lambda: ops.probe_mfma_i8(pattern, iters)] * 3)
-        return round(ops.PROBE_MFMA_OPS_PER_ITERATION * iters / (us * 1e-6) / 1e12, 1)
-
-    sustained = {"zeros": matrix_rate(0), "int4_codes_x16": matrix_rate(1), "random_bytes": matrix_rate(2)}
 
     def time_quant(x, mode, reps=20):
         return timed([lambda: ops.rotate_and_quantize_i4(x, hadamard=mode)] * reps)
@@ -526,6 +519,7 @@ def main():
     # rotation as the reference's model uses them, the seven linears, RoPE, torch's attention, residuals), module by
     # module as the reference sequences it and in the fused form (same codes; see tests/test_gpu_decoder_layer.py)
     from flh_amd.quantized_model import W4A4DecoderLayer, rotary_tables
+    from flh_amd.nn import LinearFLH
     gen = torch.Generator(device="cpu").manual_seed(11)
     lw = {n: (torch.randn(shape, generator=gen) / shape[1] ** 0.5).half().to(dev)
           for n, shape in (("q_proj", (4096, 4096)), ("k_proj", (4096, 4096)), ("v_proj", (4096, 4096)),
@@ -556,6 +550,66 @@ def main():
             layer_fig[f"token_configuration,prefill_8x512,{label}_us"] = round(wall_us(lambda: layer(xs8, cos8, sin8), reps=20), 1)
             del layer
     del lw, xs, xs8
+
+    # The Llama-3-8B decode step (32 layers, batch x 1 token, attention over 2048 cached positions, grouped queries 32 / 8,
+    # intermediate 14336 with the 28 x 512 online rotation, group-of-128 weight scales, fp16 head of 128 256 rows), random
+    # weights, captured into one graph and replayed.  Only the int4 linears and their quantisers are this library's
+    # kernels; embedding, RoPE, cache write, attention, residual adds, SiLU, the final norm and the head are stock torch
+    # ops and are reported separately (whole step minus the same step's linears-only graph).  Lower bound of the step:
+    # all int4 weights and scales + the fp16 head + the cached keys / values once over HBM.
+    from flh_amd.quantized_model import LlamaShape, W4A4LlamaModel
+    decode_model = {}
+    if not args.no_decode_model:
+        shape5 = LlamaShape.llama3_8b(num_layers=32)
+        with torch.no_grad():
+            model5 = W4A4LlamaModel.random_init(shape5, activation="token", weight_group_size=128, fused=True, seed=1)
+        w_bytes = 32 * int(sum(n * k // 2 + n * (k // 128) * 2 for _, n, k, _ in L3))
+        head_bytes = shape5.vocab_size * shape5.hidden_size * 2
+        for batch in (1, 8, 16):
+            kv_bytes = 32 * 2 * batch * shape5.num_kv_heads * 2048 * shape5.head_dim * 2
+            graph5, st5 = model5.capture_decode_step(batch, 2048)
+            for i in range(32):
+                st5["cache"].keys[i].normal_()
+                st5["cache"].values[i].normal_()
+            ms = wall_us(graph5.replay, reps=30) / 1e3
+            bound_ms = (w_bytes + head_bytes + kv_bytes) / (PEAK_HBM_GBS * 1e9) * 1e3
+            # the linears (and their quantisers) of the same step alone, as a graph over the model's own modules
+            xb5 = torch.randn(batch, 4096, dtype=torch.float16, device=dev)
+            xm5 = torch.randn(batch, 14336, dtype=torch.float16, device=dev)
+
+            def linears_only():
+                for layer in model5.layers:
+                    nw = layer._norm_weight16("input_layernorm", layer.input_layernorm)
+                    q5, s5 = ops.rmsnorm_rotate_and_quantize_i4(xb5, nw, 1e-5)
+                    LinearFLH.forward_many([layer.q_proj, layer.k_proj, layer.v_proj], q5, s5)
+                    if batch <= 2:
+                        layer.o_proj.forward_online(xb5, hadamard="exact")
+                    else:
+                        q5, s5 = ops.rotate_and_quantize_i4(xb5, hadamard="exact")
+                        layer.o_proj(q5, s5, None, x_is_packed=True)
+                    q5, s5 = ops.rmsnorm_rotate_and_quantize_i4(xb5, nw, 1e-5)
+                    LinearFLH.forward_many([layer.gate_proj, layer.up_proj], q5, s5)
+                    q5, s5 = ops.rotate_and_quantize_i4(xm5, hadamard="fast")
+                    layer.down_proj(q5, s5, None, x_is_packed=True)
+
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side), torch.no_grad():
+                linears_only()
+            torch.cuda.current_stream().wait_stream(side)
+            torch.cuda.synchronize()
+            graph_l = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph_l), torch.no_grad():
+                linears_only()
+            ms_lin = wall_us(graph_l.replay, reps=30) / 1e3
+            decode_model[f"batch={batch}"] = {
+                "ms_per_step_graph_replay": round(ms, 3), "hbm_lower_bound_ms": round(bound_ms, 3),
+                "frac_of_bound": round(bound_ms / ms, 4),
+                "linears_and_quantisers_ms": round(ms_lin, 3), "torch_ops_ms": round(ms - ms_lin, 3),
+                "linears_GB/s": round(w_bytes / (ms_lin * 1e-3) / 1e9, 1),
+                "linears_frac_hbm": round(w_bytes / (ms_lin * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
+                "bytes": {"int4_weights_and_scales": w_bytes, "fp16_head": head_bytes, "kv_cache_read": kv_bytes}}
+            del graph5, st5, graph_l
+        del model5
 
     # the same linears at the other token counts of the configuration: decode (weight streaming,
     # judged against HBM bandwidth) and a short prefill
@@ -634,9 +688,7 @@ def main():
                      "traffic": GEMM_TRAFFIC_BYTES if M == 2048 else None,
                      "avg_launch_us": round(gemm_us / len(LAYERS), 2),
                      "per_launch_us": {name: round(med[("gemm", name)], 2) for name, *_ in LAYERS},
-                     # beside the published peak: a loop of the matrix instruction alone, by operand values
-                     "matrix_instruction_alone_TOPS": sustained,
-                     "frac_of_matrix_instruction_alone_on_int4_codes": round(gemm_tops / sustained["int4_codes_x16"], 4)},
+                     },
         "roofline_hadamard_quant": {"bound": "hbm",
                                     "kernel": ("rotate_quant_mfma4096_kernel" if had_mode(4096) == "fast" else
                                                "rotate_quant_wave_kernel<8>") + f" (K=4096, M={M}, inside the step)",
@@ -652,6 +704,7 @@ def main():
         "gemm_on_6bit_matrix_instruction": f6,
         "decode_step_M=1": decode,
         "decoder_layer_llama2_7b": layer_fig,
+        "llama3_8b_decode_step_32_layers,kv_len=2048": decode_model,
         f"llama3_8b_block_M={M},weight_groups_of_128": llama3,
         "llama3_8b_decode_linears,weight_groups_of_128": llama3_decode,
         "vendor_gemm_reference": vendor,

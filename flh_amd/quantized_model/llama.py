@@ -60,6 +60,7 @@ class W4A4LlamaModel(torch.nn.Module):
             model.embed_tokens.weight.normal_(0.0, 1.0, generator=gen)
             model.lm_head.weight.normal_(0.0, 1.0 / math.sqrt(shape.hidden_size), generator=gen)
             model.norm.weight.uniform_(0.5, 1.5, generator=gen)
+            model.norm.weight.copy_(model.norm.weight.half().float())     # as a checkpoint's fp16 norm weight would be
             kv = shape.num_kv_heads * shape.head_dim
             dims = {"q_proj": (shape.hidden_size, shape.hidden_size), "k_proj": (kv, shape.hidden_size),
                     "v_proj": (kv, shape.hidden_size), "o_proj": (shape.hidden_size, shape.hidden_size),
