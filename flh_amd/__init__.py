@@ -7,6 +7,8 @@ so that existing code can switch by importing ``flh_amd`` under the name ``flh``
 the C ABI of ``libflh_hip.so``; there is no CPU or torch fallback for them -- using an op
 without the built library raises :class:`flh_amd._lib.FLHLibraryError`.
 """
+import os
+import pathlib
 import sys
 import types
 
@@ -18,12 +20,24 @@ from . import _lib
 class _LazyOps(types.ModuleType):
     """Stands where the reference has the compiled ``flh._CUDA`` module.  The HIP library
     is loaded on first attribute access, so importing the package works on a machine
-    without it (e.g. to use the torch-side helpers); calling an op there fails loudly."""
+    without it (e.g. to use the torch-side helpers); calling an op there fails loudly.
+    With the PyTorch-ROCm extension built (flh_amd/_flh_torch.so) the ops are its C++ functions
+    (``_ext_ops``); without it, or with FLH_OPS=ctypes in the environment, the ctypes route
+    (``_ops``).  Both call the same C ABI of libflh_hip.so -- neither is a fallback off the GPU."""
+
+    _impl = None
 
     def __getattr__(self, name):
-        _lib.load()  # raises FLHLibraryError with build instructions when missing
-        from . import _ops
-        return getattr(_ops, name)
+        impl = _LazyOps._impl
+        if impl is None:
+            _lib.load()  # raises FLHLibraryError with build instructions when missing
+            ext = pathlib.Path(__file__).with_name("_flh_torch.so")
+            if ext.exists() and os.environ.get("FLH_OPS", "") != "ctypes":
+                from . import _ext_ops as impl
+            else:
+                from . import _ops as impl
+            _LazyOps._impl = impl
+        return getattr(impl, name)
 
 
 _CUDA = _LazyOps("flh_amd._CUDA")

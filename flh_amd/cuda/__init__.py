@@ -7,13 +7,13 @@ from .. import _lib
 
 def load_flh_cuda_ext():
     """Reference: flh/cuda/load_ext.py:11-47 (JIT-builds and returns the extension).
-    Here the kernels are prebuilt into libflh_hip.so; this returns the op module and raises
-    when there is no GPU or no library."""
+    Here the kernels are prebuilt into libflh_hip.so; this returns the op module (the same
+    object as flh._CUDA) and raises when there is no GPU or no library."""
     if not torch.cuda.is_available():
         raise RuntimeError("CUDA not available")
     _lib.load()
-    from .. import _ops
-    return _ops
+    import flh_amd
+    return flh_amd._CUDA
 
 
 def _require(x, width=None):

@@ -254,3 +254,18 @@ def test_checkpoint_round_trip_in_the_reference_layout(tmp_path):
                                  "down_proj": LinearFLH(128, 32, group_size=128), "norm": torch.nn.LayerNorm(8)})
     with pytest.raises(ValueError, match="do not fit"):
         load_quantized(wrong, tmp_path / "ckpt")
+
+
+def test_torch_extension_loads_and_checks_tensors_without_a_device():
+    """The PyTorch-ROCm extension imports on a machine without a GPU, registers its dispatcher ops, and its tensor
+    checks reject CPU tensors before anything touches the device."""
+    ext = pytest.importorskip("flh_amd._flh_torch")
+    for name in ("gemm_i4_dequant_o16", "gemm_i4_dequant_o16_gs", "hadamard_transform_half", "hadamard_transform_64_half",
+                 "hadamard_transform_32_half", "hadamard_and_quantize_i4", "quant_and_pack_i4",
+                 "hadamard_and_quantize_i4_gs", "quant_and_pack_i4_gs"):      # flh_cuda_bindings.cpp:301-313
+        assert hasattr(ext, name) and hasattr(torch.ops.flh_hip, name)
+    a, s = torch.zeros(2, 64, dtype=torch.uint8), torch.zeros(2, 1, dtype=torch.float16)
+    with pytest.raises(RuntimeError, match="CUDA"):
+        ext.gemm_i4_dequant_o16(a, a, s, s)
+    with pytest.raises(RuntimeError, match="CUDA"):
+        ext.quant_and_pack_i4(torch.zeros(2, 128, dtype=torch.float16))
