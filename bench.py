@@ -218,6 +218,27 @@ def main():
                        for d, n in zip(qkv, "qkv"))
     del qkv, pq, ps
 
+    # ... and with gate and up as ONE launch that stores only silu(gate) * up (gemm_i4_swiglu): what a SwiGLU MLP needs
+    # in front of the down_proj rotation, without the two fp16 [M, 11008] intermediates and torch's two elementwise
+    # kernels.  Same seven contractions, six GEMM launches.
+    def step_swiglu():
+        packed = {name: ops.rotate_and_quantize_i4(acts[name], hadamard=had_mode(SOURCES[name])) for name in SOURCES}
+        for name, n, k, src in LAYERS:
+            if name in ("gate", "up"):
+                continue
+            out = ops.gemm_i4_dequant_o16(packed[src][0], weights[name][0], packed[src][1], weights[name][1])
+        return ops.gemm_i4_swiglu(packed["mlp_in"][0], weights["gate"][0], weights["up"][0], packed["mlp_in"][1],
+                                  weights["gate"][1], weights["up"][1])
+
+    for _ in range(args.warmup):
+        step_swiglu()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step_swiglu()
+    torch.cuda.synchronize()
+    ms_swiglu = (time.perf_counter() - t0) / args.steps * 1e3
+
     def timed(calls):
         """median duration in us over `calls` (a list of thunks, each one launch): HIP events on the
         launch stream around each launch, with a few GEMMs queued first so that the host runs ahead of
@@ -234,6 +255,22 @@ def main():
             pairs.append((e0, e1))
         torch.cuda.synchronize()
         return float(np.median([a.elapsed_time(b) * 1e3 for a, b in pairs]))
+
+    pq_m, ps_m = ops.rotate_and_quantize_i4(acts["mlp_in"], hadamard=had_mode(4096))
+    wg_, wu_ = weights["gate"], weights["up"]
+
+    def unfused_mlp_front():
+        g_ = ops.gemm_i4_dequant_o16(pq_m, wg_[0], ps_m, wg_[1])
+        u_ = ops.gemm_i4_dequant_o16(pq_m, wu_[0], ps_m, wu_[1])
+        return torch.nn.functional.silu(g_) * u_
+
+    swiglu = {"us_per_layer": round(ms_swiglu * 1e3, 1),
+              "TOPS": round(sum(gemm_ops(M, n, k) for _, n, k, _ in LAYERS) / (ms_swiglu * 1e-3) / 1e12, 2),
+              "gate_up_one_launch_us": round(timed([lambda: ops.gemm_i4_swiglu(pq_m, wg_[0], wu_[0], ps_m, wg_[1], wu_[1])] * 20), 2),
+              "gate_up_two_launches_plus_torch_silu_mul_us": round(timed([unfused_mlp_front] * 10), 2),
+              "launches": "4 rotate-quantise + 5 GEMM + 1 gate/up GEMM that stores silu(gate) * up only"}
+    swiglu["gate_up_one_launch_TOPS"] = round(2 * gemm_ops(M, 11008, 4096) / (swiglu["gate_up_one_launch_us"] * 1e-6) / 1e12, 1)
+    del pq_m, ps_m
 
     def time_quant(x, mode, reps=20):
         return timed([lambda: ops.rotate_and_quantize_i4(x, hadamard=mode)] * reps)
@@ -714,6 +751,7 @@ def main():
                                        "launches": "4 rotate-quantise + 4 GEMM; q/k/v and gate/up as several weight "
                                                    "matrices of one launch, weights stored separately",
                                        "equal_to_separate_launches": bool(shared_equal)},
+        "gate_up_swiglu_in_one_launch": swiglu,
         "concatenated_qkv_gate_up": {"us_per_layer": round(ms_concat * 1e3, 1),
                                      "TOPS": round(total_ops / (ms_concat * 1e-3) / 1e12, 2),
                                      "launches": "4 rotate-quantise + 4 GEMM (N = 12288, 4096, 22016, 4096)"},

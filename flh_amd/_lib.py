@@ -21,6 +21,8 @@ _SIG = {
     "flh_init": (_c.c_int, []),
     "flh_gemm_i4_o16": (_c.c_int, [_PTR, _PTR, _PTR, _PTR, _PTR, _c.c_size_t, _c.c_size_t, _c.c_size_t,
                                    _c.c_int, _c.c_int, _c.c_int, _PTR]),
+    "flh_gemm_i4_swiglu_o16": (_c.c_int, [_PTR, _PTR, _PTR, _PTR, _PTR, _PTR, _PTR, _c.c_size_t, _c.c_size_t, _c.c_size_t,
+                                          _c.c_int, _c.c_int, _c.c_int, _PTR]),
     "flh_gemm_i4_o16_multi": (_c.c_int, [_PTR, _PTR, _c.c_int, _PTR, _PTR, _PTR, _PTR, _c.c_size_t, _c.c_size_t,
                                          _c.c_int, _c.c_int, _c.c_int, _PTR]),
     "flh_rotate_quant_gemm_i4_o16_multi": (_c.c_int, [_PTR, _c.c_int, _PTR, _PTR, _PTR, _PTR, _c.c_size_t, _c.c_size_t,

@@ -110,6 +110,26 @@ def gemm_i4_dequant_multi(A, Bs, A_scale, B_scales, group_size=128):
     return Ds
 
 
+def gemm_i4_swiglu(A, B_gate, B_up, A_scale, gate_scale, up_scale, group_size=128):
+    """fp16(fp16(silu(gate)) * up) with gate / up = gemm_i4_dequant(A, B_gate / B_up, A_scale, gate_scale / up_scale),
+    in one launch that never stores gate and up: A [M, K/2], B_gate / B_up [N, K/2], scales as gemm_i4_dequant
+    (group-scaled operands: groups of 128) -> fp16 [M, N]."""
+    _check_gemm_inputs(A, B_gate, A_scale, gate_scale)
+    _check_gemm_inputs(A, B_up, A_scale, up_scale)
+    _check(B_up.shape == B_gate.shape and up_scale.shape == gate_scale.shape, "gate and up must have the same shapes")
+    M, Kp = A.shape
+    N, K = B_gate.size(0), Kp * 2
+    _check(A_scale.dim() == 2 and gate_scale.dim() == 2, "scale must be 2D")
+    _check(A_scale.size(0) == M and gate_scale.size(0) == N, "scale rows must match M / N")
+    _check(K % 128 == 0, "K must be a multiple of 128")
+    D = torch.empty((M, N), dtype=torch.float16, device=A.device)
+    if M and N:
+        _run("flh_gemm_i4_swiglu_o16", A.device, A.data_ptr(), B_gate.data_ptr(), B_up.data_ptr(), A_scale.data_ptr(),
+             gate_scale.data_ptr(), up_scale.data_ptr(), D.data_ptr(), M, N, K, A_scale.size(1), gate_scale.size(1),
+             int(group_size), _stream(A))
+    return D
+
+
 def gemm_i4_dequant_o16(A, B, A_scale, B_scale):
     """flh_cuda_bindings.cpp:75-113.  Scales are [M, K/128] and [N, K/128]; as an
     extension a width of 1 means one scale per row."""

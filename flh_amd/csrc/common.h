@@ -36,6 +36,15 @@ __device__ __forceinline__ float round_here(float v) {
   return v;
 }
 
+// fp16( float(fp16(silu(gate))) * float(up) ): the two roundings of torch's fp16 silu followed by its fp16 multiply
+// (the product the reference's MLP hands to the quantiser of down_proj, flh/quantized_model/modeling_llama.py:522-526);
+// silu in float32 as g * rcp(1 + exp(-g)) on the hardware exponential and reciprocal
+__device__ __forceinline__ _Float16 silu_mul_f16(_Float16 gate, _Float16 up) {
+  const float g = (float)gate;
+  const _Float16 act = (_Float16)round_here(g * __builtin_amdgcn_rcpf(1.0f + __expf(-g)));
+  return (_Float16)round_here((float)act * (float)up);
+}
+
 // 16 bytes per lane from global memory straight into LDS: lane i of the wave writes
 // lds_base + 16 * i (lds_base wave-uniform).  Counted by vmcnt; the compiler does not know
 // about it, so every wait for these loads is written out by hand below.

@@ -247,9 +247,7 @@ __global__ __launch_bounds__(256) void silu_mul_group_kernel(const __half* __res
   h2 v[4];
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
-    const float g = (float)g8[i];
-    const _Float16 act = (_Float16)round_here(g * __builtin_amdgcn_rcpf(1.0f + __expf(-g)));
-    const _Float16 prod = (_Float16)round_here((float)act * (float)u8[i]);
+    const _Float16 prod = silu_mul_f16(g8[i], u8[i]);
     if (i & 1) v[i >> 1].y = prod;
     else v[i >> 1].x = prod;
   }

@@ -31,6 +31,9 @@ struct GemmArgs {
   const uint8_t* seg_B[kMaxGemmSegments];
   const __half* seg_Bs[kMaxGemmSegments];
   void* seg_D[kMaxGemmSegments];
+  // SwiGLU launches (gate = B / Bs, up = B2 / Bs2, N = channels of each, D [M, N] = fp16(fp16(silu(gate)) * up))
+  const uint8_t* B2;
+  const __half* Bs2;
 };
 
 // Small-M (decode) kernels: weight-streaming, split over K inside a workgroup.

@@ -85,7 +85,13 @@ __device__ __forceinline__ void interleave_hint() {
 // through LDS.  This doubles / quadruples the waves per SIMD when a problem has only about
 // one tile per compute unit, so that one wave's unpack work overlaps another's MFMAs; integer
 // addition keeps the result bit-identical.  With KS == 2 each quad finishes half of the rows.
-template <int BM, int BN, int WM, int WN, int STAGES, int EPI, int GROUP = 128, int KS = 1>
+//
+// SWIGLU: the launch computes gate = A . Bg^T and up = A . Bu^T for the SAME output channels in one workgroup and stores
+// fp16(fp16(silu(gate)) * up) only.  The tile's BN weight rows are BN/2 rows of the gate matrix followed by the same
+// BN/2 rows of the up matrix, so the waves of the left half of the tile hold gate values and those of the right half
+// the matching up values; both halves go through the epilogue's fp16 staging tiles in LDS (rounded to fp16 exactly as
+// the two separate GEMMs would store them), where each wave then combines half of the rows.
+template <int BM, int BN, int WM, int WN, int STAGES, int EPI, int GROUP = 128, int KS = 1, bool SWIGLU = false>
 __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN) * KS, (KS == 1 && WM * WN <= 128 * 64) ? FLH_GEMM_OCC : 1)
 void gemm_i4_kernel(const GemmArgs p) {
   constexpr bool GROUPED = EPI == kGroupScale || EPI == kTokenGroup;
@@ -102,6 +108,8 @@ void gemm_i4_kernel(const GemmArgs p) {
   static_assert(EPI == kInt32 || (BM / WM) * (BN / WN) * WM * EPI_PITCH <= KS * STAGES * STAGE,
                 "epilogue staging must fit the ring");
   static_assert(KS == 1 || (!GROUPED && (KS - 1) * BM * BN * 4 <= KS * STAGES * STAGE), "K split");
+  static_assert(!SWIGLU || (KS == 1 && EPI != kInt32 && BN / WN == 2), "gate | up halves are the two wave columns");
+  constexpr int BNC = SWIGLU ? BN / 2 : BN;           // output channels per tile
   constexpr int ES = (KS == 2 && TM % 2 == 0) ? 2 : 1;   // quads that take part in the epilogue
   constexpr int TE = TM / ES;                            // 32-row blocks of a wave tile finished per quad
 
@@ -137,7 +145,7 @@ void gemm_i4_kernel(const GemmArgs p) {
       wN = p.seg_N[s];
       seg_tile = tile_n - p.seg_tile0[s];
     }
-  const int m0 = tile_m * BM, n0 = seg_tile * BN;
+  const int m0 = tile_m * BM, n0 = seg_tile * BNC;
   const int Kb = p.K >> 1;                            // bytes per packed row
 
   // per-lane byte offsets of this wave's NI load instructions inside A resp. B (stage 0); rows past
@@ -145,16 +153,17 @@ void gemm_i4_kernel(const GemmArgs p) {
   // a wave-uniform base (matrix + K position) in scalar registers plus this 32-bit offset, so a
   // stage costs no vector address arithmetic.
   unsigned voff[NI];
-  bool from_a[NI];
+  int src_of[NI];                                      // 0: activations, 1: weights, 2: the up matrix (SWIGLU)
 #pragma unroll
   for (int i = 0; i < NI; ++i) {
     const int slot = (wave * NI + i) * 64 + lane;
-    const bool isA = __builtin_amdgcn_readfirstlane(slot < BM * 4);   // a 64-slot group never straddles A | B
+    const bool isA = __builtin_amdgcn_readfirstlane(slot < BM * 4);   // a 64-slot group (16 rows) never straddles A | B
     const int r = (isA ? slot : slot - BM * 4) >> 2;
     const int c = (slot & 3) ^ ((r >> 2) & 3);
-    const int gr = isA ? min(m0 + r, p.M - 1) : min(n0 + r, wN - 1);
+    const bool second = SWIGLU && !isA && __builtin_amdgcn_readfirstlane(r >= BNC);   // ... nor gate | up
+    const int gr = isA ? min(m0 + r, p.M - 1) : min(n0 + (second ? r - BNC : r), wN - 1);
     voff[i] = (unsigned)gr * (unsigned)Kb + c * 16;
-    from_a[i] = isA;
+    src_of[i] = isA ? 0 : second ? 2 : 1;
   }
   // stages of this quad: the K steps are dealt out as evenly as possible, the first quads take the remainder
   const int KTall = p.K / (2 * kStageBytes), kt_base = KTall / KS, kt_rem = KTall % KS;
@@ -166,8 +175,9 @@ void gemm_i4_kernel(const GemmArgs p) {
     const unsigned base = lds0 + stage * STAGE + wave * NI * 1024;
     const uint8_t* ka = p.A + (size_t)k * kStageBytes;
     const uint8_t* kb = wB + (size_t)k * kStageBytes;
+    const uint8_t* kb2 = SWIGLU ? p.B2 + (size_t)k * kStageBytes : kb;
 #pragma unroll
-    for (int i = 0; i < NI; ++i) load_to_lds16(from_a[i] ? ka : kb, voff[i], base + i * 1024);
+    for (int i = 0; i < NI; ++i) load_to_lds16(src_of[i] == 0 ? ka : src_of[i] == 1 ? kb : kb2, voff[i], base + i * 1024);
   };
 
   v16i acc[TM][TN];
@@ -239,8 +249,11 @@ void gemm_i4_kernel(const GemmArgs p) {
   unsigned short sraw[8];
   const bool sc_thread = tid < SCROWS;
   const int sc_cols = tid < BM ? p.a_cols : p.b_cols;
+  const int sc_brow = min(tid, SCROWS - 1) - BM;      // weight row of the tile this thread fetches scales for
+  const bool sc_second = SWIGLU && sc_brow >= BNC;
   const __half* const sc_src = (tid < BM ? p.As + (size_t)min(m0 + tid, p.M - 1) * p.a_cols
-                                         : wBs + (size_t)min(n0 + min(tid, SCROWS - 1) - BM, wN - 1) * p.b_cols);
+                                         : (sc_second ? p.Bs2 : wBs) +
+                                               (size_t)min(n0 + (sc_second ? sc_brow - BNC : sc_brow), wN - 1) * p.b_cols);
   // Ordinary loads: the compiler's own wait for them is "everything outstanding", which is what the top
   // of the next iteration waits for anyway with a three-stage ring -- so they are requested at the end
   // of one iteration and stored at the top of the next.
@@ -296,9 +309,10 @@ void gemm_i4_kernel(const GemmArgs p) {
 #pragma unroll
     for (int i = 0; i < (BM + BN + QT * KS - 1) / (QT * KS); ++i) {
       const int e = tid + i * QT * KS;
-      const int m = m0 + e, n = n0 + e - BM;
+      const bool second = SWIGLU && e - BM >= BNC;
+      const int m = m0 + e, n = n0 + e - BM - (second ? BNC : 0);
       scale_reg[i] = e < BM ? (m < p.M ? p.As[m] : __float2half(1.f))
-                            : (e < BM + BN && n < wN ? wBs[n] : __float2half(1.f));
+                            : (e < BM + BN && n < wN ? (second ? p.Bs2 : wBs)[n] : __float2half(1.f));
     }
   }
   if constexpr (GROUPED) sc_issue(0);
@@ -511,11 +525,40 @@ void gemm_i4_kernel(const GemmArgs p) {
           *(h4*)(ep + (i * 32 + frag_row) * EPI_PITCH + nl * 2) = v;
         }
       }
-    // ... and write it out as whole row segments (the tile is private to the wave: no barrier)
     constexpr int CPR = WN / 8;                        // 16-byte chunks per row of the wave tile
     constexpr int RPI = 64 / CPR;                      // rows per store instruction
     const int crow = lane / CPR, cchunk = lane % CPR;
     const bool vec_ok = (wN & 7) == 0;
+    if constexpr (SWIGLU) {
+      // the gate tile (left wave column) and the up tile (right wave column) of this row band are both in LDS after
+      // the barrier; each of the two waves combines half of the band's rows and stores 16-byte runs of the product
+      __syncthreads();
+      const int wcol = wave % WAVES_N;
+      const uint8_t* gate_t = lds + (wave - wcol) * (TE * 32 * EPI_PITCH);
+      const uint8_t* up_t = gate_t + TE * 32 * EPI_PITCH;
+#pragma unroll
+      for (int it = 0; it < TE * 32 / (2 * RPI); ++it) {
+        const int row = wcol * (TE * 16) + it * RPI + crow;
+        const int m = m0 + wm + row, n = n0 + cchunk * 8;
+        const h8 g8 = *(const h8*)(gate_t + row * EPI_PITCH + cchunk * 16);
+        const h8 u8 = *(const h8*)(up_t + row * EPI_PITCH + cchunk * 16);
+        h8 o;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) o[e] = silu_mul_f16(g8[e], u8[e]);
+        if (m < p.M) {
+          __half* dst = (__half*)wD + (size_t)m * wN + n;
+          if (vec_ok && n + 8 <= wN) {
+            *(h8*)dst = o;
+          } else {
+            const __half* hv = (const __half*)&o;
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+              if (n + e < wN) dst[e] = hv[e];
+          }
+        }
+      }
+    } else {
+    // ... and write it out as whole row segments (the tile is private to the wave: no barrier)
 #pragma unroll
     for (int it = 0; it < TE * 32 / RPI; ++it) {
       const int row = it * RPI + crow;
@@ -533,6 +576,7 @@ void gemm_i4_kernel(const GemmArgs p) {
         }
       }
     }
+    }
   }
 }
 
@@ -543,10 +587,11 @@ int total_n(const GemmArgs& a) {
   return n;
 }
 
-template <int BM, int BN, int WM, int WN, int STAGES, int EPI, int GROUP = 128, int KS = 1>
+template <int BM, int BN, int WM, int WN, int STAGES, int EPI, int GROUP = 128, int KS = 1, bool SWIGLU = false>
 int launch(GemmArgs a, hipStream_t stream) {
+  constexpr int BNC = SWIGLU ? BN / 2 : BN;           // output channels per tile
   a.tiles_m = (a.M + BM - 1) / BM;
-  a.tiles_n = (a.N + BN - 1) / BN;
+  a.tiles_n = (a.N + BNC - 1) / BNC;
   for (int s = 1; s < a.n_seg; ++s) {                 // further weight matrices: their tiles follow
     a.seg_tile0[s] = a.tiles_n;
     a.tiles_n += (a.seg_N[s] + BN - 1) / BN;
@@ -555,7 +600,7 @@ int launch(GemmArgs a, hipStream_t stream) {
   // the ring(s), plus the tile's fp16 scales (one per row, or two blocks of eight groups per row)
   const size_t smem = (size_t)KS * STAGES * (BM + BN) * kStageBytes +
                       (EPI == kRowScale ? (BM + BN) * 2 : (EPI == kGroupScale || EPI == kTokenGroup) ? (BM + BN) * 32 : 0);
-  auto kern = gemm_i4_kernel<BM, BN, WM, WN, STAGES, EPI, GROUP, KS>;
+  auto kern = gemm_i4_kernel<BM, BN, WM, WN, STAGES, EPI, GROUP, KS, SWIGLU>;
   static std::atomic<bool> attr_set{false};   // set-up is idempotent: a race only repeats it  // per instantiation
   if (!attr_set.load(std::memory_order_acquire)) {
     if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess)
@@ -635,6 +680,25 @@ int gemm_dispatch(GemmArgs a, int epi, int group, hipStream_t stream) {
   }
 }
 
+// SwiGLU launches: tile by the number of 128-column tiles of [gate | up] together; no K split (the epilogue pairs the
+// two wave columns of a workgroup)
+template <int EPI>
+int launch_swiglu(const GemmArgs& a, int group, hipStream_t stream) {
+  auto tiles = [&](int bm) { return (long)((a.M + bm - 1) / bm) * ((a.N + 63) / 64); };
+  int tile = tiles(256) > 256 ? 256 : tiles(128) >= 256 ? 128 : 64;
+  const int forced = g_tune_tile.load(std::memory_order_relaxed);
+  if (forced == 256 || forced == 128 || forced == 64) tile = forced;
+  if constexpr (EPI == kRowScale) {
+    if (tile == 256) return launch<256, 128, 128, 64, FLH_GEMM_STAGES, EPI, 128, 1, true>(a, stream);
+    if (tile == 128) return launch<128, 128, 64, 64, 3, EPI, 128, 1, true>(a, stream);
+    return launch<64, 64, 32, 32, 3, EPI, 128, 1, true>(a, stream);
+  } else {
+    (void)group;                                       // groups of 128 only
+    if (tile >= 128) return launch<128, 128, 64, 64, 3, EPI, 128, 1, true>(a, stream);
+    return launch<64, 64, 32, 32, 3, EPI, 128, 1, true>(a, stream);
+  }
+}
+
 int check_common(const void* A, const void* B, const void* D, size_t M, size_t N, size_t K) {
   if ((M && N) && (!A || !B || !D)) return fail(FLH_EINVAL, "gemm: null pointer");
   if (misaligned16(A, B, D)) return fail(FLH_EINVAL, "gemm: A, B and D must be 16-byte aligned");
@@ -677,6 +741,29 @@ extern "C" int flh_gemm_i4_o16(const uint8_t* A, const uint8_t* B, const flh_hal
   }
   GemmArgs g{A, B, (const __half*)a_scale, (const __half*)b_scale, D, (int)M, (int)N, (int)K, a_cols, b_cols, 0, 0, 0};
   return gemm_dispatch(g, grouped ? kGroupScale : kRowScale, group, (hipStream_t)stream);
+}
+
+extern "C" int flh_gemm_i4_swiglu_o16(const uint8_t* A, const uint8_t* B_gate, const uint8_t* B_up, const flh_half* a_scale,
+                                      const flh_half* gate_scale, const flh_half* up_scale, flh_half* D, size_t M, size_t N,
+                                      size_t K, int a_cols, int b_cols, int group, void* stream) {
+  if (int e = check_common(A, B_gate, D, M, N, K)) return e;
+  if ((M && N) && !B_up) return fail(FLH_EINVAL, "gemm: null pointer");
+  if (misaligned16(B_up)) return fail(FLH_EINVAL, "gemm: A, B and D must be 16-byte aligned");
+  if (M == 0 || N == 0) return FLH_OK;
+  if (!a_scale || !gate_scale || !up_scale) return fail(FLH_EINVAL, "gemm: null scale pointer");
+  const bool grouped = a_cols != 1 || b_cols != 1;
+  if (grouped) {
+    if (group != 128) return fail(FLH_EINVAL, "gemm (SwiGLU): group-scaled operands need groups of 128, not %d", group);
+    const int ng = (int)(K / 128);
+    if ((a_cols != 1 && a_cols != ng) || (b_cols != 1 && b_cols != ng))
+      return fail(FLH_EINVAL, "gemm: scale columns (%d, %d) must be 1 or K/group = %d", a_cols, b_cols, ng);
+  }
+  GemmArgs g{A, B_gate, (const __half*)a_scale, (const __half*)gate_scale, D, (int)M, (int)N, (int)K, a_cols, b_cols, 0, 0, 0};
+  g.B2 = B_up;
+  g.Bs2 = (const __half*)up_scale;
+  if (!grouped) return launch_swiglu<kRowScale>(g, group, (hipStream_t)stream);
+  if (a_cols == 1) return launch_swiglu<kTokenGroup>(g, group, (hipStream_t)stream);
+  return launch_swiglu<kGroupScale>(g, group, (hipStream_t)stream);
 }
 
 extern "C" int flh_gemm_i4_o16_multi(const uint8_t* A, const flh_half* a_scale, int count, const uint8_t* const* B,

@@ -110,6 +110,22 @@ Tensor gemm_i4_dequant_o16_gs(const Tensor& A, const Tensor& B, const Tensor& A_
   return gemm_checked(A, B, A_scale, B_scale, group_size);
 }
 
+// gate and up projection of a SwiGLU MLP in one launch: fp16(fp16(silu(gate)) * up)
+Tensor gemm_i4_swiglu(const Tensor& A, const Tensor& B_gate, const Tensor& B_up, const Tensor& A_scale,
+                      const Tensor& gate_scale, const Tensor& up_scale, int64_t group_size) {
+  check_gemm_inputs(A, B_gate, A_scale, gate_scale);
+  check_gemm_inputs(A, B_up, A_scale, up_scale);
+  TORCH_CHECK(B_up.sizes() == B_gate.sizes() && up_scale.sizes() == gate_scale.sizes(),
+              "gate and up must have the same shapes");
+  const int64_t M = A.size(0), N = B_gate.size(0), K = A.size(1) * 2;
+  Tensor D = torch::empty({M, N}, A_scale.options());
+  if (M == 0 || N == 0) return D;
+  Launch l(A);
+  ok(flh_gemm_i4_swiglu_o16(u8(A), u8(B_gate), u8(B_up), h(A_scale), h(gate_scale), h(up_scale), hm(D), M, N, K,
+                            (int)A_scale.size(1), (int)gate_scale.size(1), (int)group_size, stream_of(A)));
+  return D;
+}
+
 std::vector<Tensor> gemm_i4_dequant_multi(const Tensor& A, const std::vector<Tensor>& Bs, const Tensor& A_scale,
                                           const std::vector<Tensor>& B_scales, int64_t group_size) {
   TORCH_CHECK(Bs.size() == B_scales.size() && !Bs.empty() && Bs.size() <= 4,
@@ -376,6 +392,8 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         py::arg("group_size") = 128);
   m.def("gemm_i4_dequant_multi", &gemm_i4_dequant_multi, py::arg("A"), py::arg("Bs"), py::arg("A_scale"),
         py::arg("B_scales"), py::arg("group_size") = 128);
+  m.def("gemm_i4_swiglu", &gemm_i4_swiglu, py::arg("A"), py::arg("B_gate"), py::arg("B_up"), py::arg("A_scale"),
+        py::arg("gate_scale"), py::arg("up_scale"), py::arg("group_size") = 128);
   m.def("rotate_quantize_gemm_i4", &rotate_quantize_gemm_i4, py::arg("x"), py::arg("B"), py::arg("B_scale"));
   m.def("rotate_quantize_gemm_i4_multi", &rotate_quantize_gemm_i4_multi, py::arg("x"), py::arg("Bs"), py::arg("B_scales"));
   m.def("hadamard_transform_half", &hadamard_transform_half, py::arg("x"));

@@ -113,6 +113,27 @@ class LinearFLH(torch.nn.Module):
                                            a_rows, w_scales, group)
         return [(y if l.bias is None else y + l.bias).view(*lead, l.out_features) for y, l in zip(ys, layers)]
 
+    @staticmethod
+    def forward_swiglu(gate_layer, up_layer, x, a_scale):
+        """act_fn(gate_layer(x)) * up_layer(x) of a SwiGLU MLP (flh/quantized_model/modeling_llama.py:522-526) in one
+        GEMM launch that stores only the product: x packed codes [..., K/2], a_scale as for forward.  The two
+        projections are rounded to fp16 as their own calls would store them, then combined as torch's fp16 silu and
+        multiply do (the device's exponential: the fp16 result can differ from torch's in its last bit in a few values
+        per thousand)."""
+        if (gate_layer.in_features != up_layer.in_features or gate_layer.out_features != up_layer.out_features
+                or gate_layer.w_scale.shape != up_layer.w_scale.shape):
+            raise ValueError("forward_swiglu: gate and up must have the same shape and weight-scale layout")
+        if gate_layer.bias is not None or up_layer.bias is not None:
+            raise ValueError("forward_swiglu: layers with a bias take the separate calls")
+        lead = x.shape[:-1]
+        rows = x.view(-1, x.size(-1))
+        n, k = gate_layer.out_features, gate_layer.in_features
+        group = gate_layer.weight_group_size if gate_layer.weight_group_size > 0 else (gate_layer.in_group_size or 128)
+        y = _pkg._CUDA.gemm_i4_swiglu(rows, gate_layer.w_packed.view(n, k // 2), up_layer.w_packed.view(n, k // 2),
+                                      a_scale.reshape(rows.size(0), -1), gate_layer.w_scale.view(n, -1),
+                                      up_layer.w_scale.view(n, -1), group)
+        return y.view(*lead, n)
+
     def forward_online(self, x, hadamard=True):
         """fp16 activations [..., K] -> fp16 [..., N] with the activation side done here: whole-row rotation
         (`hadamard`: as in rotate_and_quantize_i4), one symmetric int4 scale per token, then the GEMM -- the

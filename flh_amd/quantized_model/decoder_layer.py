@@ -236,6 +236,11 @@ class W4A4DecoderLayer(torch.nn.Module):
         self._tap("o_proj", y)
         return y, cache
 
+    def _swiglu_gemm_applies(self):
+        g = self.gate_proj
+        cols = g.w_scale.view(g.out_features, -1).size(1)
+        return g.bias is None and self.up_proj.bias is None and (cols == 1 or (g.weight_group_size == 128 and cols == g.in_features // 128))
+
     def _group_quant(self, stage, quantizer, x):
         s, z, q = quantizer(x)
         self._tap(stage + ".input", x.reshape(-1, x.size(-1)))
@@ -246,6 +251,11 @@ class W4A4DecoderLayer(torch.nn.Module):
     def mlp(self, x):
         s, z, q = self._norm_quant("mlp_in", self.post_attention_layernorm, "post_attention_layernorm",
                                    self.mlp_quantizer1, x)
+        if (self.activation == "token" and self.fused and self.record is None and q.numel() // q.size(-1) > 64
+                and self._swiglu_gemm_applies()):
+            # prefill: gate and up in one launch that stores silu(gate) * up only (no fp16 [M, I] round trips)
+            s, z, q = self._token_quant("mlp_mid", LinearFLH.forward_swiglu(self.gate_proj, self.up_proj, q, s))
+            return self.down_proj(q, s, z, x_is_packed=True)
         gate, up = self._project([self.gate_proj, self.up_proj], q, s, z)
         self._tap("gate_proj", gate), self._tap("up_proj", up)
         if self.activation == "token":

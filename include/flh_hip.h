@@ -72,6 +72,19 @@ int flh_gemm_i4_o16_multi(const uint8_t* A, const flh_half* a_scale, int count, 
                           const flh_half* const* b_scale, flh_half* const* D, const size_t* N, size_t M, size_t K,
                           int a_cols, int b_cols, int group, void* stream);
 
+/* The gate and up projections of a SwiGLU MLP in one launch that stores only their combination:
+ *   D[m, c] = fp16( float(fp16(silu(gate[m, c]))) * float(up[m, c]) ),  silu(g) = g / (1 + exp(-g)) in float32,
+ * where gate = flh_gemm_i4_o16(A, B_gate, a_scale, gate_scale, ...) and up = the same with B_up / up_scale, both
+ * [M, N] and rounded to fp16 exactly as those calls would store them -- D is what the reference's MLP computes with
+ * two GEMM calls and two torch kernels, act_fn(gate_proj(x)) * up_proj(x) (flh/quantized_model/modeling_llama.py:522-526),
+ * before it quantises the product for down_proj.  A workgroup computes the same output channels of both matrices, so
+ * the two fp16 [M, N] intermediates never go to memory.  Scale layouts as flh_gemm_i4_o16 (group-scaled operands:
+ * groups of 128 only).  The exponential and the reciprocal are the device's: against a float64 evaluation the fp16
+ * result differs in its last bit in fewer than 2e-3 of the values. */
+int flh_gemm_i4_swiglu_o16(const uint8_t* A, const uint8_t* B_gate, const uint8_t* B_up, const flh_half* a_scale,
+                           const flh_half* gate_scale, const flh_half* up_scale, flh_half* D, size_t M, size_t N,
+                           size_t K, int a_cols, int b_cols, int group, void* stream);
+
 /* Decode: flh_rotate_quant_i4 (float32 butterflies, one scale per token) and flh_gemm_i4_o16 in ONE launch, for one
  * to four tokens: x [M, 4096] fp16 (M <= 4), B [N, 2048], b_scale [N, b_cols] with b_cols = 1 or 32 -> D [M, N] fp16.
  * Every workgroup rotates and quantises the tokens itself (the additions of the stand-alone kernel in the same
