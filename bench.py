@@ -17,12 +17,13 @@ dominant kernel (the GEMM, against the dense int8 MFMA peak), the roofline of th
 Hadamard-quant kernel (against HBM bandwidth), and the CPU oracle timed on a bounded
 sample of the same workload.
 
-Rotation modes (--hadamard): "mixed" (default) runs the bit-exact float32-butterfly kernel for
-the power-of-two rows (K = 4096) and the matrix-core kernel for K = 11008 = 172 x 64, whose
-dense factor has no reference-defined summation order; "exact" / "fast" force one mode for all
-four launches.  Both modes are timed per kernel and reported either way.
+Rotation modes (--hadamard): "fast" (default) runs the matrix-core kernels for all four launches: K = 4096 differs
+from the float32-butterfly codes in fewer than 1e-5 of the positions (measured live and reported; it is closer to the
+reference's float64 transform than the float32 butterflies are), K = 11008 = 172 x 64 in about 4e-4 (no summation
+order is defined by the reference for its dense factor).  "mixed" runs the bit-exact float32-butterfly kernel for
+K = 4096, "exact" for all four.  All modes are timed per kernel and reported either way.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline] [--hadamard mixed]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline] [--hadamard fast]
 """
 import argparse
 import json
@@ -105,7 +106,7 @@ def main():
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also launch three elementwise passes over 256 MiB (read 256 MiB, write 256 MiB): the "
                          "known-size kernel that hardware-counter readings (FETCH_SIZE / WRITE_SIZE) are scaled by")
-    ap.add_argument("--hadamard", choices=["mixed", "exact", "fast"], default="mixed")
+    ap.add_argument("--hadamard", choices=["mixed", "exact", "fast"], default="fast")
     ap.add_argument("--large-tokens", type=int, default=16384,
                     help="token count of the extra Hadamard-quant launches that amortise the launch floor")
     args = ap.parse_args()
@@ -114,7 +115,9 @@ def main():
                  "cross-GPU part; run with --gpus 1")
 
     import torch
-    from flh_amd import _ops as ops
+    import flh_amd
+    from flh_amd import synthetic as syn
+    ops = flh_amd._CUDA           # the PyTorch-ROCm extension in front of the C ABI (ctypes ops where it has no wrapper)
     if not torch.cuda.is_available():
         sys.exit("bench.py needs the MI355X (no CPU fallback for the product path)")
     M = args.tokens
@@ -338,14 +341,59 @@ def main():
         del gate, up
     del xl
 
-    # cold variant of the memory-bound kernel: 24 distinct inputs (403 MB, more than the 256 MB last-level
-    # cache) visited in turn, so that no launch finds its input on chip
-    cold_in = [torch.from_numpy(acts_h["attn_in"]).to(dev) for _ in range(24)]
+    # Cold inputs, timed without host gaps: a graph of launches over distinct input / output buffers that together exceed
+    # the 256 MB last-level cache (no launch finds its rows on chip), replayed; per-launch time = replay / launches.
+    # For every shape: the float32-butterfly mode, the matrix-core mode, the same kernel without rotation (quantise only)
+    # and a plain device copy of the same fp16 rows -- the two streaming floors a rotation kernel can be held against.
+    def graph_us(fns, reps=10):
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for f in fns:
+                f()
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            for f in fns:
+                f()
+        g.replay()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            g.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e3 / reps / len(fns)
+
+    side = torch.cuda.Stream()
     cold = {}
-    for mode in ("exact", "fast"):
-        us = timed([(lambda x=x: ops.rotate_and_quantize_i4(x, hadamard=mode)) for x in cold_in])
-        cold[mode] = {"us": round(us, 2), "GB/s": round(quant_bytes(M, 4096) / (us * 1e-6) / 1e9, 1)}
-    del cold_in
+    for k_c, m_c in ((4096, M), (11008, M), (14336, M), (4096, ML)):
+        n_buf = max(4, int(300e6 // (m_c * k_c * 2)) + 1)
+        base = torch.from_numpy(syn.activations(min(m_c, 2048), k_c, seed=k_c)).to(dev)
+        xs_c = [base.repeat(m_c // base.size(0), 1) if m_c > base.size(0) else base.clone() for _ in range(n_buf)]
+        ys_c = [torch.empty_like(x) for x in xs_c[:2]]
+        row = {"distinct_inputs": n_buf, "algorithmic_bytes": quant_bytes(m_c, k_c)}
+        for label, fn in (("fast", lambda x, i: ops.rotate_and_quantize_i4(x, hadamard="fast")),
+                          ("exact", lambda x, i: ops.rotate_and_quantize_i4(x, hadamard="exact")),
+                          ("quantise_only", lambda x, i: ops.rotate_and_quantize_i4(x, hadamard=False)),
+                          ("device_copy", lambda x, i: ys_c[i % 2].copy_(x))):
+            if label == "exact" and k_c != 4096 and m_c > 2048:
+                continue
+            us = graph_us([(lambda x=x, i=i: fn(x, i)) for i, x in enumerate(xs_c)])
+            byts = 2 * 2 * m_c * k_c if label == "device_copy" else quant_bytes(m_c, k_c)
+            row[label] = {"us": round(us, 2), "GB/s": round(byts / (us * 1e-6) / 1e9, 1),
+                          "frac_hbm": round(byts / (us * 1e-6) / 1e9 / PEAK_HBM_GBS, 4)}
+        row["fast_over_quantise_only"] = round(row["fast"]["us"] / row["quantise_only"]["us"], 3)
+        cold[f"K={k_c},M={m_c}"] = row
+        del xs_c, ys_c, base
+    # how far the matrix-core mode is from the float32-butterfly codes (K = 4096: both against each other on the device)
+    qe_, se_ = ops.rotate_and_quantize_i4(acts["attn_in"], hadamard="exact")
+    qf_, sf_ = ops.rotate_and_quantize_i4(acts["attn_in"], hadamard="fast")
+    nib = lambda t: torch.stack((t & 15, t >> 4), -1)
+    cold["K=4096:fast_vs_exact_code_mismatch_rate"] = float((nib(qe_) != nib(qf_)).float().mean())
+    cold["K=4096:fast_vs_exact_scale_mismatch_rate"] = float((se_ != sf_).float().mean())
+    del qe_, se_, qf_, sf_
 
     # decode (M = 1): the whole step is launch-bound, so it is also recorded into a graph once and replayed
     # (the library allocates nothing and needs no set-up after flh_init, so it can be captured as it is)
@@ -367,7 +415,6 @@ def main():
         torch.cuda.synchronize()
         return (time.perf_counter() - t0) / reps * 1e6
 
-    side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
     with torch.cuda.stream(side):
         decode_step()
@@ -465,7 +512,6 @@ def main():
 
     # the Llama-3-8B block of the same path: group-wise weight scales (g = 128), one activation scale per token, grouped
     # queries (k / v 1024 wide), intermediate 14336 with the 28 x 512 online rotation; per layer, weights on the device
-    from flh_amd import synthetic as syn
     L3 = [("q", 4096, 4096, "attn_in"), ("k", 1024, 4096, "attn_in"), ("v", 1024, 4096, "attn_in"), ("o", 4096, 4096, "attn_out"),
           ("gate", 14336, 4096, "mlp_in"), ("up", 14336, 4096, "mlp_in"), ("down", 4096, 14336, "mlp_mid")]
     L3_SRC = {"attn_in": 4096, "attn_out": 4096, "mlp_in": 4096, "mlp_mid": 14336}
