@@ -215,11 +215,6 @@ __global__ __launch_bounds__(256) void rotate_quant_mfma4096_kernel(const __half
 template <int DT>
 struct DenseFactor;
 template <>
-struct DenseFactor<2> {                           // K = 4096: the factor across blocks is H64 itself
-  static constexpr int D = 64;
-  __device__ static bool plus(int r, int c) { return !(__builtin_popcount(r & c) & 1); }
-};
-template <>
 struct DenseFactor<6> {
   static constexpr int D = 172;
   __device__ static bool plus(int r, int c) {   // M[r][c] = had172[r][c]
@@ -252,7 +247,6 @@ __global__ void build_dense_fragments(h8* table) {
   table[frag * 64 + lane] = v;
 }
 
-static __device__ h8 g_frag64[2 * 2 * 2 * 64];
 static __device__ h8 g_frag172[2 * 6 * 6 * 64];
 static __device__ h8 g_frag224[2 * 7 * 7 * 64];
 
@@ -505,9 +499,7 @@ int dense_table(const h8** out) {
     if (!t) {
       constexpr int NFRAG = 2 * DT * DT;
       void* sym = nullptr;
-      const hipError_t e = DT == 2   ? hipGetSymbolAddress(&sym, HIP_SYMBOL(g_frag64))
-                           : DT == 6 ? hipGetSymbolAddress(&sym, HIP_SYMBOL(g_frag172))
-                                     : hipGetSymbolAddress(&sym, HIP_SYMBOL(g_frag224));
+      const hipError_t e = DT == 6 ? hipGetSymbolAddress(&sym, HIP_SYMBOL(g_frag172)) : hipGetSymbolAddress(&sym, HIP_SYMBOL(g_frag224));
       if (e != hipSuccess) return fail(FLH_ELAUNCH, "rotate_quant: cannot locate the factor table: %s", hipGetErrorString(e));
       hipLaunchKernelGGL((build_dense_fragments<DT>), dim3(NFRAG), dim3(64), 0, nullptr, (h8*)sym);
       if (int rc = check_launch("build_dense_fragments")) return rc;
@@ -538,9 +530,7 @@ int launch_dense(const __half* x, uint8_t* q, __half* scales, uint32_t M, float 
       return fail(FLH_ELAUNCH, "rotate_quant: cannot reserve %zu bytes of LDS", smem);
     attr[split].store(true, std::memory_order_release);
   }
-  // resident workgroups: one per compute unit with the large factor tables in LDS, two with the 8 KB table of K = 4096
-  const unsigned cap = DT == 2 ? 512u : 256u;
-  const unsigned blocks = split ? M : ((M + 3) / 4 < cap ? (M + 3) / 4 : cap);
+  const unsigned blocks = split ? M : ((M + 3) / 4 < 256u ? (M + 3) / 4 : 256u);
   hipLaunchKernelGGL(kern, dim3(blocks), dim3(kThreadsDense), smem, stream, x, q, scales, table, M,
                      1.0f / sqrtf((float)K), clip);
   return check_launch("rotate_quant_mfma_dense");
@@ -553,15 +543,13 @@ bool rotate_quant_mfma_supports(uint32_t K) { return K == 4096 || K == 11008 || 
 // one-time set-up of the matrix-core kernels (called by flh_init)
 int rotate_quant_mfma_init() {
   const h8* t = nullptr;
-  if (int rc = dense_table<2>(&t)) return rc;
   if (int rc = dense_table<6>(&t)) return rc;
   return dense_table<7>(&t);
 }
 
 // launcher used by flh_rotate_quant_i4 (fwht_quant.hip)
 int launch_rotate_quant_mfma(const __half* x, uint8_t* q, __half* scales, uint32_t M, uint32_t K, float clip,
-                             hipStream_t stream, bool pairs) {
-  if (K == 4096 && pairs) return launch_dense<2>(x, q, scales, M, clip, stream);
+                             hipStream_t stream) {
   if (K == 11008) return launch_dense<6>(x, q, scales, M, clip, stream);
   if (K == 14336) return launch_dense<7>(x, q, scales, M, clip, stream);
   if (K != 4096) return fail(FLH_EINVAL, "rotate_quant (matrix-core mode): K = %u is not supported", K);

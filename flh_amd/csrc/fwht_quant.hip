@@ -650,7 +650,7 @@ int launch_rmsnorm(const __half* x, const __half* w, uint8_t* q, __half* s, uint
 
 // matrix-core variant (fwht_mfma.hip)
 int launch_rotate_quant_mfma(const __half* x, uint8_t* q, __half* scales, uint32_t M, uint32_t K, float clip,
-                             hipStream_t stream, bool pairs);
+                             hipStream_t stream);
 bool rotate_quant_mfma_supports(uint32_t K);
 
 }  // namespace flh
@@ -768,9 +768,9 @@ extern "C" int flh_rotate_quant_i4(const flh_half* x, uint8_t* q_packed, flh_hal
   __half* sh = (__half*)scales;
   __half* yh = (__half*)y_out;
 
-  if (hadamard == FLH_HAD_MFMA || hadamard == 3) {
+  if (hadamard == FLH_HAD_MFMA) {
     if (had_group <= 0 && scale_group == 0 && !y_out && rotate_quant_mfma_supports(K))
-      return launch_rotate_quant_mfma(xh, q_packed, sh, M, K, clip_ratio, st, hadamard == 3);
+      return launch_rotate_quant_mfma(xh, q_packed, sh, M, K, clip_ratio, st);
     hadamard = FLH_HAD_F32;  // shapes / options the matrix-core kernels do not cover
   }
   int Kd = 1, P = 1;

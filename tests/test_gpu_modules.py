@@ -331,3 +331,37 @@ def test_hql_linear4bit_alias(g):
     assert np.allclose(y.astype(np.float64), ref.astype(np.float64), rtol=1e-3, atol=1e-2)
     full = x.astype(np.float64) @ w.astype(np.float64).T
     assert np.linalg.norm(y - full) / np.linalg.norm(full) < 0.3
+
+
+def test_checkpoint_load_gives_the_same_forward_bits(tmp_path):
+    """A tree of LinearFLH layers saved in the reference's layout (model.pt in pickle protocol 4 +
+    quantization_config.json) and loaded into a freshly built tree on the GPU: the same forward bits, also on the
+    6-bit path whose second encoding of the weights is rebuilt after the load."""
+    from flh_amd.nn import load_quantized, save_quantized
+    torch.manual_seed(5)
+
+    def tree(fill):
+        mk = lambda k, n: (LinearFLH.from_float(torch.nn.Linear(k, n, bias=False).half(), weight_group_size=128,
+                                                in_group_size=128, no_hadamard=True) if fill
+                           else LinearFLH(k, n, in_group_size=128, group_size=128))
+        return torch.nn.ModuleDict({"up": mk(512, 384), "down": mk(384, 512)})
+
+    src = tree(True).cuda()
+    x = dev(syn.activations(300, 512, seed=2))
+    quant = ActQuantizer(bits=4, group_size=128, use_hadamard=False, packed_output=True)
+
+    def run(model):
+        s, z, q = quant(x)
+        h = model["up"](q, s, z, x_is_packed=True)
+        s, z, q = quant(h)
+        return h, model["down"](q, s, z, x_is_packed=True)
+    want = run(src)
+    save_quantized(src, tmp_path / "ckpt")
+    dst = tree(False)
+    dst["up"].six_bit = True
+    dst = dst.cuda()
+    before = run(dst)                                    # zero weights: builds the 6-bit encoding of the empty layer
+    assert float(before[1].abs().max()) == 0.0
+    load_quantized(dst, tmp_path / "ckpt", device="cuda")
+    got = run(dst)
+    assert torch.equal(got[0], want[0]) and torch.equal(got[1], want[1])

@@ -240,7 +240,8 @@ def test_checkpoint_round_trip_in_the_reference_layout(tmp_path):
     cfg = json.loads((tmp_path / "ckpt" / "quantization_config.json").read_text())
     assert cfg == {"weight_bits": 4, "weight_group_size": 128, "act_bits": 4, "act_group_size": 128,
                    "weight_sym": True, "act_sym": True, "clip_ratio": 0.9, "dtype": "float16"}
-    stored = torch.load(tmp_path / "ckpt" / "model.pt", weights_only=True)
+    from flh_amd.nn.checkpoint import read_state_dict
+    stored = read_state_dict(tmp_path / "ckpt" / "model.pt")
     assert stored["norm.weight"].dtype == torch.float16 and stored["q_proj.w_packed"].dtype == torch.uint8
     dst = tree(False)
     got = load_quantized(dst, tmp_path / "ckpt")
@@ -254,6 +255,42 @@ def test_checkpoint_round_trip_in_the_reference_layout(tmp_path):
                                  "down_proj": LinearFLH(128, 32, group_size=128), "norm": torch.nn.LayerNorm(8)})
     with pytest.raises(ValueError, match="do not fit"):
         load_quantized(wrong, tmp_path / "ckpt")
+
+
+def test_state_dict_reader_takes_the_references_pickle_protocol_and_nothing_else(tmp_path):
+    """The reference writes model.pt with pickle protocol 4 (flh/quantized_model/modeling_llama.py:1107), which
+    torch's non-executing loader refuses; the allow-list reader returns the same tensors (shared storages, offsets and
+    non-contiguous views included) and refuses a file that names any other global."""
+    import collections
+    import pickle
+    from flh_amd.nn.checkpoint import read_state_dict
+    base = torch.arange(48, dtype=torch.float16)
+    state = collections.OrderedDict(
+        packed=torch.randint(0, 256, (37, 5), dtype=torch.uint8), scale=torch.rand(7, 3).half(),
+        view=base[8:32].view(4, 6), strided=base.view(6, 8).t(), other=base, i64=torch.arange(5), empty=torch.zeros(0, 4).half(),
+        b=torch.tensor([True, False]), f32=torch.rand(3))
+    for proto in (2, 4):
+        path = tmp_path / f"m{proto}.pt"
+        torch.save(state, path, pickle_protocol=proto)
+        got = read_state_dict(path)
+        assert list(got) == list(state)
+        for k, v in state.items():
+            assert got[k].dtype == v.dtype and got[k].shape == v.shape and torch.equal(got[k], v), (proto, k)
+    with pytest.raises(pickle.UnpicklingError):
+        torch.load(tmp_path / "m4.pt", weights_only=True)        # the reason the reader exists
+
+    class Evil:
+        def __reduce__(self):
+            import os
+            return (os.getcwd, ())
+    bad = tmp_path / "bad.pt"
+    torch.save({"x": torch.zeros(2), "y": Evil()}, bad, pickle_protocol=4)
+    with pytest.raises(pickle.UnpicklingError, match="refused"):
+        read_state_dict(bad)
+    notdict = tmp_path / "list.pt"
+    torch.save([torch.zeros(2)], notdict, pickle_protocol=4)
+    with pytest.raises(pickle.UnpicklingError):
+        read_state_dict(notdict)
 
 
 def test_torch_extension_loads_and_checks_tensors_without_a_device():
