@@ -19,6 +19,7 @@ gemm_i4_dequant_o16 = _ext.gemm_i4_dequant_o16
 gemm_i4_dequant_o16_gs = _ext.gemm_i4_dequant_o16_gs
 gemm_i4_dequant_multi = _ext.gemm_i4_dequant_multi
 gemm_i4_swiglu = _ext.gemm_i4_swiglu
+rope_kv_cache_ = _ext.rope_kv_cache_
 rotate_quantize_gemm_i4 = _ext.rotate_quantize_gemm_i4
 rotate_quantize_gemm_i4_multi = _ext.rotate_quantize_gemm_i4_multi
 hadamard_transform_half = _ext.hadamard_transform_half

@@ -53,6 +53,8 @@ _SIG = {
     "quant_and_pack_host": (None, [_PTR, _PTR, _PTR, _c.c_uint32]),
     "had_and_quant_host_gs": (None, [_c.c_int, _PTR, _PTR, _PTR, _c.c_uint32]),
     "quant_and_pack_host_gs": (None, [_c.c_int, _PTR, _PTR, _PTR, _c.c_uint32]),
+    "flh_rope_kv_cache_f16": (_c.c_int, [_PTR, _PTR, _PTR, _PTR, _PTR, _PTR, _PTR, _PTR, _c.c_uint32, _c.c_uint32,
+                                         _c.c_uint32, _c.c_uint32, _c.c_uint32, _c.c_uint32, _PTR]),
     "flh_fwht_f16_inplace": (_c.c_int, [_PTR, _c.c_uint32, _c.c_int, _PTR]),
     "flh_rotate_quant_i4": (_c.c_int, [_PTR, _PTR, _PTR, _PTR, _c.c_uint32, _c.c_uint32, _c.c_int, _c.c_int,
                                        _c.c_int, _c.c_float, _PTR]),

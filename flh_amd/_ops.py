@@ -337,6 +337,30 @@ def gemm_f6_int32(A6, B6):
     return C
 
 
+def rope_kv_cache_(q, k, v, cos, sin, positions, k_cache, v_cache):
+    """Rotary embedding of q (in place) and k, and the new keys / values written into their cache slots, one launch:
+    q [B, T, Hq, d], k / v [B, T, Hkv, d] fp16 contiguous; cos / sin [T, d] fp16; positions [T] int64 on the device;
+    k_cache / v_cache [B, Hkv, max_len, d] fp16 contiguous.  The arithmetic of q * cos + rotate_half(q) * sin evaluated
+    operation by operation in fp16.  Returns q."""
+    for t_ in (q, k, v, cos, sin, k_cache, v_cache):
+        _check(t_.is_cuda and t_.dtype == torch.float16 and t_.is_contiguous() and t_.device == q.device,
+               "tensors must be contiguous float16 CUDA tensors on one device")
+    _check(q.dim() == 4 and k.dim() == 4 and v.shape == k.shape and k.shape[:2] == q.shape[:2] and k.size(3) == q.size(3),
+           "q [B, T, Hq, d] and k, v [B, T, Hkv, d] expected")
+    B, T, Hq, d = q.shape
+    Hkv = k.size(2)
+    _check(cos.shape == (T, d) and sin.shape == (T, d), "cos / sin must be [T, d]")
+    _check(positions.is_cuda and positions.dtype == torch.int64 and positions.is_contiguous() and positions.numel() == T
+           and positions.device == q.device, "positions must be a contiguous int64 CUDA tensor of T entries")
+    _check(k_cache.dim() == 4 and k_cache.shape == v_cache.shape and k_cache.size(0) == B and k_cache.size(1) == Hkv
+           and k_cache.size(3) == d, "caches must be [B, Hkv, max_len, d]")
+    _check(d % 16 == 0, "head_dim must be a multiple of 16")
+    if q.numel():
+        _run("flh_rope_kv_cache_f16", q.device, q.data_ptr(), k.data_ptr(), v.data_ptr(), cos.data_ptr(), sin.data_ptr(),
+             positions.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), B, T, Hq, Hkv, d, k_cache.size(2), _stream(q))
+    return q
+
+
 def _check_rows(x, width):
     _check(x.is_cuda, "Input tensor must be on CUDA")
     _check(x.dtype == torch.float16, "Input tensor must be float16 (half)")

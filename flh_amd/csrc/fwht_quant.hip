@@ -572,6 +572,17 @@ __global__ __launch_bounds__(512) void rotate_quant_row8_kernel(const __half* __
   const size_t row = blockIdx.x;
   rotate_quant_row_8waves(x + row * 4096, stage, wave_max8, q + row * 2048, scales + row, norm, wave);
 }
+// ... and with RMSNorm in front (flh_rmsnorm_rotate_quant_i4), the same bytes as rotate_quant_wave_kernel<8, ..., RMS>
+__global__ __launch_bounds__(512) void rmsnorm_rotate_quant_row8_kernel(const __half* __restrict__ x,
+                                                                        const __half* __restrict__ weight, float eps,
+                                                                        uint8_t* __restrict__ q,
+                                                                        __half* __restrict__ scales, float norm) {
+  __shared__ float stage[8 * 8 * 64];
+  __shared__ float wave_max8[8];
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const size_t row = blockIdx.x;
+  rotate_quant_row_8waves<true>(x + row * 4096, stage, wave_max8, q + row * 2048, scales + row, norm, wave, weight, eps);
+}
 // measured per launch inside a replayed graph: 2.7 against 4.4 us for one row, 3.2 against 4.9 us for 256 rows,
 // 3.9 against 5.0 us for 512; from 1024 rows on the wave-per-row kernel is the faster one
 constexpr uint32_t kRow8MaxRows = 512;
@@ -717,6 +728,10 @@ extern "C" int flh_rmsnorm_rotate_quant_i4(const flh_half* x, const flh_half* we
   __half *sh = (__half*)scales, *yh = (__half*)y_out;
   const bool had = hadamard != FLH_HAD_NONE;
   hipStream_t st = (hipStream_t)stream;
+  if (had && K == 4096 && !yh && clip_ratio >= 1.0f && M <= kRow8MaxRows && (!wh || !misaligned16(wh))) {
+    hipLaunchKernelGGL(rmsnorm_rotate_quant_row8_kernel, dim3(M), dim3(512), 0, st, xh, wh, eps, q_packed, sh, 1.0f / 64.0f);
+    return check_launch("rmsnorm_rotate_quant_row8");
+  }
   switch (K / 512) {
     case 1: return launch_wave_rms<1>(xh, wh, eps, q_packed, sh, yh, M, had, clip_ratio, st);
     case 2: return launch_wave_rms<2>(xh, wh, eps, q_packed, sh, yh, M, had, clip_ratio, st);

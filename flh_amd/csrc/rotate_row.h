@@ -221,11 +221,47 @@ __device__ __forceinline__ void rotate_quant_row(const __half* __restrict__ x_ro
 // strides 512, 1024, 2048 run across the waves through LDS (stage: 8 x 8 x 64 floats, wave_max: 8 floats).
 // The same additions in the same order as rotate_quant_row<8>, hence the same codes and scale.  Every wave of the
 // workgroup must call it (four barriers).
+// RMS: the row is normalised first, as rotate_quant_row<8, ..., RMS> does it.  Every wave reads the whole row once
+// more (it is in the compute unit's cache by then) and sums the squares in exactly that routine's order -- per lane
+// over the eight 512-value segments, then the fixed tree over the lanes -- so that the statistics, the normalised
+// fp16 row and therefore the codes are bit-identical to the wave-per-row kernel's, without a pass over the waves.
+template <bool RMS = false>
 __device__ __forceinline__ void rotate_quant_row_8waves(const __half* __restrict__ x_row, float* stage, float* wave_max8,
-                                                        uint8_t* q_row, __half* scale_dst, float norm, int wave) {
+                                                        uint8_t* q_row, __half* scale_dst, float norm, int wave,
+                                                        const __half* __restrict__ rms_weight = nullptr,
+                                                        float rms_eps = 0.f) {
   const int lane = threadIdx.x & 63;
   const int c = lane_chunk(lane);
-  const v4i raw = *(const v4i*)(x_row + wave * 512 + c * 8);
+  v4i raw = *(const v4i*)(x_row + wave * 512 + c * 8);
+  if constexpr (RMS) {
+    float ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const v4i seg = *(const v4i*)(x_row + j * 512 + c * 8);
+#pragma unroll
+      for (int d = 0; d < 4; ++d) {
+        const unsigned w = (unsigned)seg[d];
+        const h2 t = __builtin_bit_cast(h2, w);
+        ss = __builtin_fmaf((float)t[0], (float)t[0], ss);
+        ss = __builtin_fmaf((float)t[1], (float)t[1], ss);
+      }
+    }
+    ss = wave_sum(ss);
+    const float inv = 1.0f / __builtin_sqrtf(ss / 4096.0f + rms_eps);
+    v4i wv = {0, 0, 0, 0};
+    if (rms_weight) wv = *(const v4i*)(rms_weight + wave * 512 + c * 8);
+#pragma unroll
+    for (int d = 0; d < 4; ++d) {
+      const unsigned w = (unsigned)raw[d], ww = (unsigned)wv[d];
+      const h2 t = __builtin_bit_cast(h2, w), g = __builtin_bit_cast(h2, ww);
+      float a = round_here((float)t[0] * inv), b = round_here((float)t[1] * inv);
+      if (rms_weight) {
+        a = round_here(a * (float)g[0]);
+        b = round_here(b * (float)g[1]);
+      }
+      raw[d] = (int)pack_f16(a, b);
+    }
+  }
   float v[8];
 #pragma unroll
   for (int d = 0; d < 4; ++d) {

@@ -359,6 +359,30 @@ std::vector<Tensor> rmsnorm_and_quantize_i4_gs(const Tensor& x, const c10::optio
   return {q, s};
 }
 
+// ---- rotary embedding + cache write -----------------------------------------------------------------------------------
+Tensor rope_kv_cache_(Tensor q, const Tensor& k, const Tensor& v, const Tensor& cos, const Tensor& sin,
+                      const Tensor& positions, Tensor k_cache, Tensor v_cache) {
+  for (const Tensor* t : std::initializer_list<const Tensor*>{&q, &k, &v, &cos, &sin, &k_cache, &v_cache})
+    TORCH_CHECK(t->is_cuda() && t->scalar_type() == torch::kFloat16 && t->is_contiguous() && t->device() == q.device(),
+                "tensors must be contiguous float16 CUDA tensors on one device");
+  TORCH_CHECK(q.dim() == 4 && k.dim() == 4 && v.sizes() == k.sizes() && k.size(0) == q.size(0) && k.size(1) == q.size(1) &&
+                  k.size(3) == q.size(3), "q [B, T, Hq, d] and k, v [B, T, Hkv, d] expected");
+  const int64_t B = q.size(0), T = q.size(1), Hq = q.size(2), d = q.size(3), Hkv = k.size(2);
+  TORCH_CHECK(cos.dim() == 2 && cos.size(0) == T && cos.size(1) == d && sin.sizes() == cos.sizes(), "cos / sin must be [T, d]");
+  TORCH_CHECK(positions.is_cuda() && positions.scalar_type() == torch::kInt64 && positions.is_contiguous() &&
+                  positions.numel() == T && positions.device() == q.device(),
+              "positions must be a contiguous int64 CUDA tensor of T entries");
+  TORCH_CHECK(k_cache.dim() == 4 && k_cache.sizes() == v_cache.sizes() && k_cache.size(0) == B && k_cache.size(1) == Hkv &&
+                  k_cache.size(3) == d, "caches must be [B, Hkv, max_len, d]");
+  TORCH_CHECK(d % 16 == 0, "head_dim must be a multiple of 16");
+  if (q.numel() == 0) return q;
+  Launch l(q);
+  ok(flh_rope_kv_cache_f16(hm(q), h(k), h(v), h(cos), h(sin), (const int64_t*)positions.data_ptr(), hm(k_cache), hm(v_cache),
+                           (uint32_t)B, (uint32_t)T, (uint32_t)Hq, (uint32_t)Hkv, (uint32_t)d, (uint32_t)k_cache.size(2),
+                           stream_of(q)));
+  return q;
+}
+
 }  // namespace
 
 // dispatcher ops (torch.ops.flh_hip.*): the reference's nine names and the general forms
@@ -396,6 +420,8 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         py::arg("gate_scale"), py::arg("up_scale"), py::arg("group_size") = 128);
   m.def("rotate_quantize_gemm_i4", &rotate_quantize_gemm_i4, py::arg("x"), py::arg("B"), py::arg("B_scale"));
   m.def("rotate_quantize_gemm_i4_multi", &rotate_quantize_gemm_i4_multi, py::arg("x"), py::arg("Bs"), py::arg("B_scales"));
+  m.def("rope_kv_cache_", &rope_kv_cache_, py::arg("q"), py::arg("k"), py::arg("v"), py::arg("cos"), py::arg("sin"),
+        py::arg("positions"), py::arg("k_cache"), py::arg("v_cache"));
   m.def("hadamard_transform_half", &hadamard_transform_half, py::arg("x"));
   m.def("hadamard_transform_128_half", &hadamard_transform_half, py::arg("x"));   // the name flh/cuda/hadamard.py:35 calls
   m.def("hadamard_transform_64_half", &hadamard_transform_64_half, py::arg("x"));

@@ -43,6 +43,30 @@ def rotary_tables(positions, head_dim, theta=10000.0, dtype=torch.float16):
     return ang.cos().to(dtype), ang.sin().to(dtype)
 
 
+def _decode_attention(q, k, v):
+    """softmax(q k^T / sqrt(d)) v for ONE query position per sequence, as three batched matrix products' worth of stock
+    tensor operations (the fused attention kernels are built for long query blocks and take 80 us for this shape):
+    q [B, H, 1, d], k / v [B, Hkv, L, d] -> [B, H, 1, d]; query heads of one key / value head form the rows of a small
+    matrix.  Scores and probabilities in float32."""
+    b, h, _, d = q.shape
+    hkv, n = k.size(1), k.size(2)
+    qg = q.reshape(b * hkv, h // hkv, d)
+    kt = k.reshape(b * hkv, n, d).transpose(1, 2)
+    global _BMM_F32_OUT
+    if _BMM_F32_OUT is None:                           # fp16 operands, float32 result, where this torch build has it
+        try:
+            torch.bmm(qg, kt, out_dtype=torch.float32)
+            _BMM_F32_OUT = True
+        except (TypeError, RuntimeError):
+            _BMM_F32_OUT = False
+    scores = torch.bmm(qg, kt, out_dtype=torch.float32) if _BMM_F32_OUT else torch.bmm(qg, kt).float()
+    probs = torch.softmax(scores * (1.0 / d ** 0.5), dim=-1).to(q.dtype)
+    return torch.bmm(probs, v.reshape(b * hkv, n, d)).reshape(b, h, 1, d)
+
+
+_BMM_F32_OUT = None
+
+
 def _rotate_half(x):
     half = x.size(-1) // 2
     return torch.cat((-x[..., half:], x[..., :half]), dim=-1)
@@ -63,10 +87,11 @@ class StaticKVCache:
         def __init__(self, owner, index):
             self.owner, self.index = owner, index
 
-        def update(self, k, v, positions):
+        def rope_and_update(self, q, k, v, cos, sin, positions):
+            """q [B, T, Hq, d] (rotated in place), k / v [B, T, Hkv, d] of the new tokens -> the first kv_len slots of
+            this layer's keys / values, the new ones (keys rotated) written at `positions`."""
             keys, values = self.owner.keys[self.index], self.owner.values[self.index]
-            keys.index_copy_(2, positions, k)
-            values.index_copy_(2, positions, v)
+            _ops().rope_kv_cache_(q, k, v, cos, sin, positions, keys, values)
             n = self.owner.kv_len
             return keys[:, :, :n], values[:, :, :n]
 
@@ -150,7 +175,7 @@ class W4A4DecoderLayer(torch.nn.Module):
     # ------------------------------------------------------------------ pieces
     def _tap(self, name, value):
         if self.record is not None:
-            self.record[name] = value
+            self.record[name] = value.clone()      # a copy: q is rotated in place later on
 
     def _norm_weight16(self, name, norm):
         """The norm weight as the fused kernels take it (fp16; exact for weights that came from an fp16 checkpoint),
@@ -204,25 +229,29 @@ class W4A4DecoderLayer(torch.nn.Module):
         s, z, q = self._norm_quant("attn_in", self.input_layernorm, "input_layernorm", self.attn_quantizer1, x)
         qs, ks, vs = self._project([self.q_proj, self.k_proj, self.v_proj], q, s, z)
         self._tap("q_proj", qs), self._tap("k_proj", ks), self._tap("v_proj", vs)
-        qs = qs.view(b, t, self.num_heads, self.head_dim).transpose(1, 2)
-        ks = ks.view(b, t, self.num_kv_heads, self.head_dim).transpose(1, 2)
-        vs = vs.view(b, t, self.num_kv_heads, self.head_dim).transpose(1, 2)
-        qs = qs * cos + _rotate_half(qs) * sin
-        ks = ks * cos + _rotate_half(ks) * sin
         static = isinstance(kv_cache, StaticKVCache._Layer)
         if static:
-            ks, vs = kv_cache.update(ks, vs, positions)
+            # rotary embedding of q (in place) and k, and the new keys / values into their cache slots: one launch
+            qs = qs.view(b, t, self.num_heads, self.head_dim)
+            ks, vs = kv_cache.rope_and_update(qs, ks.view(b, t, self.num_kv_heads, self.head_dim),
+                                              vs.view(b, t, self.num_kv_heads, self.head_dim), cos, sin, positions)
+            qs = qs.transpose(1, 2)
             cache = kv_cache
         else:
+            qs = qs.view(b, t, self.num_heads, self.head_dim).transpose(1, 2)
+            ks = ks.view(b, t, self.num_kv_heads, self.head_dim).transpose(1, 2)
+            vs = vs.view(b, t, self.num_kv_heads, self.head_dim).transpose(1, 2)
+            qs = qs * cos + _rotate_half(qs) * sin
+            ks = ks * cos + _rotate_half(ks) * sin
             if kv_cache is not None:
                 ks, vs = torch.cat((kv_cache[0], ks), dim=2), torch.cat((kv_cache[1], vs), dim=2)
             cache = (ks, vs)
         gqa = self.num_heads != self.num_kv_heads
         past = ks.size(2) - t
-        if past == 0:
+        if t == 1 and past > 0:
+            out = _decode_attention(qs, ks, vs)           # one new token sees every cached position
+        elif past == 0:
             out = torch.nn.functional.scaled_dot_product_attention(qs, ks, vs, is_causal=t > 1, enable_gqa=gqa)
-        elif t == 1:      # one new token sees every cached position
-            out = torch.nn.functional.scaled_dot_product_attention(qs, ks, vs, enable_gqa=gqa)
         else:
             mask = torch.ones(t, past + t, dtype=torch.bool, device=x.device).tril(diagonal=past)
             out = torch.nn.functional.scaled_dot_product_attention(qs, ks, vs, attn_mask=mask, enable_gqa=gqa)

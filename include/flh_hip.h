@@ -232,6 +232,23 @@ int flh_rotate_quant_i4(const flh_half* x, uint8_t* q_packed, flh_half* scales, 
                         uint32_t M, uint32_t K, int hadamard, int had_group, int scale_group,
                         float clip_ratio, void* stream);
 
+/* ---------------------------------------------------------------------------------
+ * Between the q / k / v GEMM and attention of a decode (or prefill) step: rotary position embedding of the query and
+ * key heads and the write of the new keys / values into a preallocated cache, one launch.  No native counterpart in the
+ * reference, whose attention calls transformers' apply_rotary_pos_emb and cache update as separate tensor operations
+ * (flh/quantized_model/modeling_llama.py:403-424).
+ *   q [B, T, Hq, d] fp16, rotated in place;  k, v [B, T, Hkv, d] fp16 (read only);
+ *   cos, sin [T, d] fp16 (the tables of the T new positions);  positions [T] int64 ON THE DEVICE (the cache slots of
+ *   the new tokens: a captured graph is replayed for other positions by overwriting this tensor);
+ *   k_cache, v_cache [B, Hkv, max_len, d] fp16: slot positions[t] receives the rotated key resp. the value of token t
+ *   (a position outside [0, max_len) writes nothing).
+ * y = fp16( fp16(x * cos) + fp16(rotate_half(x) * sin) ), rotate_half((x1, x2)) = (-x2, x1) over the two halves of a
+ * head -- the roundings of the tensor expression evaluated operation by operation in fp16.  d a multiple of 16.
+ * --------------------------------------------------------------------------------- */
+int flh_rope_kv_cache_f16(flh_half* q, const flh_half* k, const flh_half* v, const flh_half* cos, const flh_half* sin,
+                          const int64_t* positions, flh_half* k_cache, flh_half* v_cache, uint32_t B, uint32_t T,
+                          uint32_t Hq, uint32_t Hkv, uint32_t head_dim, uint32_t max_len, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

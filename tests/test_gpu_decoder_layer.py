@@ -67,8 +67,12 @@ def test_decoding_with_the_cache_matches_prefill():
         outs.append(y)
     step = torch.cat(outs, dim=1)
     assert cache[0].shape == (1, 2, t, 128)
-    # same quantised operands token by token; attention kernels differ between the two shapes
-    assert torch.allclose(step.float(), full.float(), rtol=2e-2, atol=2e-2)
+    # same quantised operands in front of attention token by token; the attention arithmetic differs between the two
+    # shapes (fused kernel / batched matrix products) in the last fp16 bits, which the o_proj quantiser can turn into a
+    # flipped code here and there: equal within the quantisation noise, token 0 (no past) bit for bit
+    assert torch.equal(step[:, 0], full[:, 0])
+    rel = (step.float() - full.float()).norm(dim=-1) / full.float().norm(dim=-1)
+    assert float(rel.max()) < 0.1 and float(rel.median()) < 0.02, rel
 
 
 def test_close_to_the_fp16_layer():

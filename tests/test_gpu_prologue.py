@@ -211,3 +211,15 @@ def test_prologue_argument_errors(ops):
         ops.rmsnorm_rotate_and_quantize_i4(torch.zeros(2, 1536, dtype=torch.float16, device="cuda"), None, 1e-5)
     q, s = ops.rmsnorm_and_quantize_i4_gs(x[:0], None, 1e-5, 128)
     assert q.shape == (0, 128) and s.shape == (0, 2)
+
+
+def test_rmsnorm_rotate_short_batches_give_the_long_batch_bytes(ops):
+    """Up to 512 rows of 4096 take one workgroup of eight waves per row, more take one wave per row: the same sums in
+    the same order (statistics included), so a row's codes and scale do not depend on the batch it arrives in."""
+    x = dev(syn.activations(700, 4096, seed=11))
+    w = dev(np.random.default_rng(12).uniform(0.5, 1.5, 4096).astype(np.float16))
+    for weight in (w, None):
+        q_long, s_long = ops.rmsnorm_rotate_and_quantize_i4(x, weight, 1e-5)
+        for rows in (1, 8, 16, 300, 512):
+            q, s = ops.rmsnorm_rotate_and_quantize_i4(x[:rows].contiguous(), weight, 1e-5)
+            assert torch.equal(q, q_long[:rows]) and torch.equal(s, s_long[:rows]), rows
