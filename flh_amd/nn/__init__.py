@@ -5,3 +5,4 @@ from .hadamard import OnlineHadamard  # noqa: F401
 from . import linear_gs, quantization_gs  # noqa: F401
 from .fused import RMSNormQuant, SiluMulQuant  # noqa: F401
 from .checkpoint import save_quantized, load_quantized  # noqa: F401
+from .gptq import FLHGPTQ, GPTQQuantizer  # noqa: F401

@@ -31,5 +31,9 @@ than "retyping the formula" fixes each function) is listed per module; the summa
                    per-token x per-channel epilogue is a closed form (one fp32
                    rounding, one fp16 rounding); group epilogue follows the reference
                    kernel's ascending-group fp32 accumulation with fused multiply-add.
+* ``layer``     -- a decoder layer / decode step composed of the pieces above with float64 rotary embedding and
+                   attention, pinned by special cases (tests/test_oracle_layer.py).
+* ``gptq``      -- GPTQ in the rotated basis in its elimination form, pinned by closed forms and properties
+                   (tests/test_oracle_gptq.py).
 """
 from . import pack, hadamard, quant, gemm, linear  # noqa: F401

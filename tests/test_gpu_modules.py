@@ -365,3 +365,33 @@ def test_checkpoint_load_gives_the_same_forward_bits(tmp_path):
     load_quantized(dst, tmp_path / "ckpt", device="cuda")
     got = run(dst)
     assert torch.equal(got[0], want[0]) and torch.equal(got[1], want[1])
+
+
+def test_gptq_on_the_gpu_matches_the_oracle():
+    """FLHGPTQ with the layer and the calibration inputs on the GPU (float32 tensor arithmetic there) against the
+    float64 elimination form of oracle/gptq.py, then packed by LinearFLH.from_float and run through the GEMM."""
+    from flh_amd.nn import FLHGPTQ
+    from oracle import gptq as OG
+    from oracle import hadamard as OH
+    rng = np.random.default_rng(6)
+    cols, rows = 512, 64
+    mix = rng.standard_normal((cols, cols)) * 2.0 / np.sqrt(cols) + np.eye(cols)
+    x = rng.standard_normal((1500, cols)) @ mix
+    w = (rng.standard_normal((rows, cols)) * 0.05).astype(np.float32)
+    layer = torch.nn.Linear(cols, rows, bias=False).cuda()
+    layer.weight.data.copy_(torch.from_numpy(w))
+    g = FLHGPTQ(layer)
+    g.add_batch(torch.from_numpy(x).float().cuda(), None, group_size=128)
+    g.fasterquant(group_size=128, actorder=True)
+    got = layer.weight.data.cpu().numpy().astype(np.float64)
+    want = OG.gptq(w.astype(np.float64), OG.hessian([x], 128), group_size=128, actorder=True)
+    scales, gsz = OG.grid_scales(OH.had_transform(w.astype(np.float64), 128), 128)
+    diff = np.abs(got - want) / np.repeat(scales, gsz, axis=1)
+    assert (diff > 0.5).mean() < 0.01 and diff.max() < 1.5
+    packed = LinearFLH.from_float(layer.half(), weight_group_size=128, in_group_size=128, no_hadamard=True)
+    xs = dev(syn.activations(40, cols, seed=1))
+    s, z, q = ActQuantizer(bits=4, group_size=128, use_hadamard=True, packed_output=True)(xs)
+    y = packed(q, s, z, x_is_packed=True)
+    full = OH.had_transform(host(xs).astype(np.float64), 128) @ got.T       # rotated inputs x rotated GPTQ weights
+    assert np.linalg.norm(host(y) - full) / np.linalg.norm(full) < 0.25
+    g.free()

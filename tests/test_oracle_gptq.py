@@ -1,0 +1,109 @@
+"""Pins of oracle/gptq.py (closed forms and properties) and the torch implementation flh_amd.nn.gptq against it on
+the CPU (the implementation runs the same tensor code on the GPU; tests/test_gpu_modules.py repeats the comparison there)."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import gptq as OG
+from oracle import hadamard as OH
+
+
+def calib(rng, n, cols, mix=0.6):
+    """correlated calibration inputs: a random mixing of Gaussian sources"""
+    a = rng.standard_normal((cols, cols)) * mix / np.sqrt(cols) + np.eye(cols)
+    return rng.standard_normal((n, cols)) @ a
+
+
+def test_hessian_is_batch_independent_and_a_closed_form():
+    rng = np.random.default_rng(0)
+    x = calib(rng, 300, 128)
+    whole = OG.hessian([x], 128)
+    parts = OG.hessian([x[:7], x[7:150].reshape(11, 13, 128), x[150:]], 128)
+    xr = OH.had_transform(x, 128)
+    assert np.allclose(whole, 2.0 / 300 * xr.T @ xr, rtol=1e-12) and np.allclose(parts, whole, rtol=1e-10)
+
+
+def test_diagonal_hessian_gives_round_to_nearest():
+    rng = np.random.default_rng(1)
+    w = rng.standard_normal((24, 256)) * 0.05
+    h = np.diag(rng.uniform(0.5, 2.0, 256))
+    for actorder in (False, True):
+        got = OG.gptq(w, h, group_size=128, actorder=actorder)
+        wr = OH.had_transform(w, 128)
+        scales, g = OG.grid_scales(wr, 128)
+        want = np.concatenate([OG.quantise_column(wr[:, i:i + 1], scales[:, i // g][:, None]) for i in range(256)], axis=1)
+        assert np.array_equal(got, want)
+    # codes live on the grid: |code| <= 8, the group maximum sits at +-7
+    codes = np.rint(got.reshape(24, 2, 128) / scales[:, :, None])
+    assert np.abs(codes).max() == 7 and np.allclose(codes * scales[:, :, None], got.reshape(24, 2, 128))
+
+
+def test_feedback_lowers_the_output_error_on_the_calibration_inputs():
+    rng = np.random.default_rng(2)
+    cols, rows = 256, 48
+    x = calib(rng, 2000, cols, mix=3.0)
+    w = rng.standard_normal((rows, cols)) * 0.05
+    h = OG.hessian([x], 128)
+    wr, xr = OH.had_transform(w, 128), OH.had_transform(x, 128)
+    ref = xr @ wr.T
+    rtn = OG.gptq(w, np.eye(cols), group_size=128, percdamp=0.0)
+    errs = {}
+    for name, q in (("rtn", rtn), ("gptq", OG.gptq(w, h, group_size=128)), ("gptq_actorder", OG.gptq(w, h, group_size=128, actorder=True))):
+        errs[name] = np.linalg.norm(xr @ q.T - ref) / np.linalg.norm(ref)
+    assert errs["gptq"] < 0.8 * errs["rtn"] and errs["gptq_actorder"] < 0.8 * errs["rtn"], errs
+
+
+@pytest.mark.parametrize("actorder", [False, True])
+@pytest.mark.parametrize("group_size,clip", [(128, 1.0), (128, 0.9), (-1, 1.0)])
+def test_torch_implementation_against_the_oracle(actorder, group_size, clip):
+    """FLHGPTQ (Cholesky factor, blocks of 128, float32) against the elimination form in float64: the same grid values
+    except where float32 rounding moves a column across a rounding boundary (then by one step, rarely)."""
+    from flh_amd.nn.gptq import FLHGPTQ
+    rng = np.random.default_rng(3)
+    cols, rows = 256, 40
+    x = calib(rng, 900, cols, mix=2.0)
+    w = (rng.standard_normal((rows, cols)) * 0.05).astype(np.float32)
+    layer = torch.nn.Linear(cols, rows, bias=False)
+    layer.weight.data.copy_(torch.from_numpy(w))
+    g = FLHGPTQ(layer)
+    for part in (x[:400], x[400:]):
+        g.add_batch(torch.from_numpy(part).float().view(2, -1, cols), None, group_size=group_size)
+    h_ref = OG.hessian([x], group_size if group_size > 0 else None)
+    assert np.allclose(g.H.numpy(), h_ref, rtol=2e-4, atol=2e-5)
+    g.fasterquant(group_size=group_size, blocksize=128, percdamp=0.01, actorder=actorder, sym=True, bits=4, clip_ratio=clip)
+    got = layer.weight.data.numpy().astype(np.float64)
+    want = OG.gptq(w.astype(np.float64), h_ref, group_size=group_size, actorder=actorder, clip_ratio=clip)
+    wr = OH.had_transform(w.astype(np.float64), group_size if group_size > 0 else None)
+    if clip < 1.0:
+        gg = group_size if group_size > 0 else cols
+        v = wr.reshape(rows, cols // gg, gg)
+        wr = np.clip(v, -np.abs(v).max(2, keepdims=True) * clip, np.abs(v).max(2, keepdims=True) * clip).reshape(rows, cols)
+    scales, gsz = OG.grid_scales(wr, group_size, 4, clip)
+    step = np.repeat(scales, gsz, axis=1)
+    diff = np.abs(got - want) / step
+    assert (diff > 0.5).mean() < 0.01, (diff > 0.5).mean()          # same grid point almost everywhere
+    assert diff.max() < 1.5                                           # and one step apart where not
+    xr = OH.had_transform(x, group_size if group_size > 0 else None)
+    base = np.linalg.norm(xr @ want.T - xr @ OH.had_transform(w.astype(np.float64), group_size if group_size > 0 else None).T)
+    mine = np.linalg.norm(xr @ got.T - xr @ OH.had_transform(w.astype(np.float64), group_size if group_size > 0 else None).T)
+    assert abs(mine - base) < 0.05 * base
+    g.free()
+
+
+def test_gptq_result_packs_through_linear_flh():
+    """The reference's flow after fasterquant (flh/quantized_model/modeling_llama.py:824-835): the layer now holds grid
+    values of the rotated basis, and LinearFLH.from_float(no_hadamard=True) packs them."""
+    from flh_amd.nn import LinearFLH
+    from flh_amd.nn.gptq import FLHGPTQ
+    rng = np.random.default_rng(4)
+    layer = torch.nn.Linear(256, 32, bias=False).half()
+    g = FLHGPTQ(layer)
+    g.add_batch(torch.from_numpy(calib(rng, 500, 256)).half(), None, group_size=128)
+    g.fasterquant(group_size=128, actorder=True)
+    packed = LinearFLH.from_float(layer, weight_group_size=128, in_group_size=128, no_hadamard=True)
+    assert packed.w_packed.dtype == torch.uint8 and packed.w_scale.shape == (32, 2)
+    # round-to-nearest of grid values: exact where a group still reaches code +-7 (the scale is re-derived from the
+    # group maximum), otherwise within half a step of the re-derived grid
+    deq = packed.get_weight().float().view(32, 2, 128)
+    step = packed.w_scale.float().view(32, 2, 1)
+    assert bool(((deq - layer.weight.data.float().view(32, 2, 128)).abs() <= 0.5 * step * 1.01 + 1e-4).all())
