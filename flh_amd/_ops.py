@@ -361,6 +361,45 @@ def rope_kv_cache_(q, k, v, cos, sin, positions, k_cache, v_cache):
     return q
 
 
+_attention_workspaces = {}      # (device index, stream handle) -> uint8 tensor: launches of one stream run in order
+
+
+def decode_attention(q, k_cache, v_cache, kv_len, scale=None, workspace=None):
+    """One new token per sequence against the first `kv_len` slots of a preallocated cache: q [B, Hq, d] fp16,
+    k_cache / v_cache [B, Hkv, max_len, d] fp16 -> [B, Hq, d] fp16 = softmax(q K^T * scale) V with float32 scores,
+    grouped queries (Hq / Hkv in {1, 2, 4, 8}), d in {64, 128}.  `workspace`: a uint8 CUDA tensor for the chunks' partial
+    results; by default one per (device, stream) is kept and grown as needed."""
+    for t_ in (q, k_cache, v_cache):
+        _check(t_.is_cuda and t_.dtype == torch.float16 and t_.is_contiguous() and t_.device == q.device,
+               "tensors must be contiguous float16 CUDA tensors on one device")
+    _check(q.dim() == 3 and k_cache.dim() == 4 and k_cache.shape == v_cache.shape and k_cache.size(0) == q.size(0)
+           and k_cache.size(3) == q.size(2), "q [B, Hq, d] and caches [B, Hkv, max_len, d] expected")
+    B, Hq, d = q.shape
+    Hkv, max_len = k_cache.size(1), k_cache.size(2)
+    _check(d in (64, 128), "head_dim must be 64 or 128")
+    _check(Hkv > 0 and Hq % Hkv == 0 and Hq // Hkv in (1, 2, 4, 8), "Hq / Hkv must be 1, 2, 4 or 8")
+    _check(0 < kv_len <= max_len, "kv_len must be in 1 .. max_len")
+    out = torch.empty_like(q)
+    if B == 0:
+        return out
+    need = int(_lib.load().flh_decode_attention_workspace_bytes(B, Hq, d, int(kv_len)))
+    if workspace is None:
+        key = (q.device.index, _stream(q))
+        workspace = _attention_workspaces.get(key)
+        if workspace is None or workspace.numel() < need:
+            _check(not torch.cuda.is_current_stream_capturing(),
+                   "decode_attention: call it once eagerly (or pass a workspace) before capturing a graph")
+            workspace = torch.empty(max(need, 1 << 20), dtype=torch.uint8, device=q.device)
+            _attention_workspaces[key] = workspace
+    else:
+        _check(workspace.is_cuda and workspace.dtype == torch.uint8 and workspace.is_contiguous()
+               and workspace.device == q.device and workspace.numel() >= need, f"workspace: {need} bytes of uint8 needed")
+    _run("flh_decode_attention_f16", q.device, q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(), B, Hq,
+         Hkv, d, int(kv_len), max_len, float(scale if scale is not None else d ** -0.5), workspace.data_ptr(),
+         workspace.numel(), _stream(q))
+    return out
+
+
 def _check_rows(x, width):
     _check(x.is_cuda, "Input tensor must be on CUDA")
     _check(x.dtype == torch.float16, "Input tensor must be float16 (half)")

@@ -1,0 +1,226 @@
+// Attention of ONE new token per sequence over a preallocated fp16 key / value cache (the decode step), with grouped
+// queries: out[b, h] = softmax(q[b, h] . K[b, h / rep]^T * scale) V[b, h / rep] over the first kv_len cache slots.
+//
+// Stands where the reference calls the flash-attn package (flh/quantized_model/modeling_llama.py:449-460,
+// _flash_attention_forward on the cached keys / values); the stock fused attention kernels are built for long query
+// blocks and take ~80 us for this shape, the same arithmetic as separate tensor operations ~30 us in five launches.
+// Here the cached positions are split into chunks, one workgroup per (sequence, key / value head, chunk): scores and
+// probabilities in float32, a partial (maximum, sum, weighted values) per chunk goes to a scratch buffer, and a second
+// small kernel combines the chunks' partials -- two launches, every key and value read once, all query heads of a
+// key / value head served by the same read.
+#include <atomic>
+
+#include "lane_ops.h"
+
+namespace flh {
+namespace {
+
+constexpr int kAttnThreads = 256;
+
+// partial of one (sequence, kv head, chunk): REP heads x (D weighted values, maximum, sum) as float
+template <int D>
+constexpr int partial_floats(int rep) { return rep * (D + 2); }
+
+template <int D, int REP, int CHUNK>
+__global__ __launch_bounds__(kAttnThreads) void decode_attention_partial_kernel(
+    const __half* __restrict__ q, const __half* __restrict__ k_cache, const __half* __restrict__ v_cache,
+    float* __restrict__ partials, uint32_t Hkv, uint32_t kv_len, uint32_t max_len, uint32_t splits, float scale) {
+  static_assert(D == 128 || D == 64, "head dimension");
+  static_assert(CHUNK == 64, "one key per lane in the softmax step");
+  constexpr int TPK = kAttnThreads / CHUNK;            // threads per key: 4
+  constexpr int CPT = D / TPK;                         // channels per thread in the score step: 32 (16)
+  __shared__ float qs[REP * D];                        // the query heads as float
+  __shared__ float sc[REP][CHUNK];                     // scores, then probabilities
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const uint32_t split = blockIdx.x % splits, bh = blockIdx.x / splits;   // bh = b * Hkv + kvh
+  const uint32_t t0 = split * CHUNK;
+  const __half* qh = q + (size_t)bh * REP * D;         // q [B, Hq, D]: the REP heads of this kv head are adjacent
+  for (int i = tid; i < REP * D; i += kAttnThreads) qs[i] = __half2float(qh[i]);
+  __syncthreads();
+
+  // scores: thread (key, part) takes CPT channels of its key
+  const int key = tid / TPK, part = tid % TPK;
+  const uint32_t t = t0 + key;
+  const bool live = t < kv_len;
+  const __half* kr = k_cache + ((size_t)bh * max_len + (live ? t : 0)) * D + part * CPT;
+  float kv[CPT];
+#pragma unroll
+  for (int c8 = 0; c8 < CPT / 8; ++c8) {
+    const h8 v = *(const h8*)(kr + c8 * 8);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) kv[c8 * 8 + e] = (float)v[e];
+  }
+  // this lane's channel pair (channel for D = 64) of every value row of the chunk, requested now: the loads travel
+  // while the scores and the softmax pieces are computed
+  const uint32_t n_live = kv_len > t0 ? min((uint32_t)CHUNK, kv_len - t0) : 0u;
+  const __half* vr = v_cache + ((size_t)bh * max_len + t0) * D;
+  float vv0[CHUNK], vv1[D == 128 ? CHUNK : 1];
+#pragma unroll
+  for (int i = 0; i < CHUNK; ++i) {
+    if constexpr (D == 128) {
+      h2 v = {(_Float16)0.f, (_Float16)0.f};
+      if ((uint32_t)i < n_live) v = *(const h2*)(vr + (size_t)i * D + 2 * lane);
+      vv0[i] = (float)v[0];
+      vv1[i] = (float)v[1];
+    } else {
+      vv0[i] = (uint32_t)i < n_live ? __half2float(vr[(size_t)i * D + lane]) : 0.f;
+    }
+  }
+#pragma unroll
+  for (int h = 0; h < REP; ++h) {
+    float s = 0.f;
+#pragma unroll
+    for (int c = 0; c < CPT; ++c) s = __builtin_fmaf(kv[c], qs[h * D + part * CPT + c], s);
+    s += dpp_f<kDppQuadXor1>(s);                       // the four threads of a key are one quad
+    s += dpp_f<kDppQuadXor2>(s);
+    if (part == 0) sc[h][key] = live ? s * scale : -INFINITY;
+  }
+  __syncthreads();
+
+  // softmax pieces of this chunk, head h by wave h (REP > 4: two heads per wave), then the weighted values:
+  // lane = a channel pair, all waves walk over the same value rows
+  float* out = partials + (size_t)blockIdx.x * partial_floats<D>(REP);
+  for (int h = wave; h < REP; h += kAttnThreads / 64) {
+    const float s = sc[h][lane];
+    const float m = wave_max(s);
+    const float p = m == -INFINITY ? 0.f : __expf(s - m);      // a chunk wholly past kv_len: nothing
+    const float l = wave_sum(p);
+    sc[h][lane] = p;
+    if (lane == 0) {
+      out[h * (D + 2) + D] = m;
+      out[h * (D + 2) + D + 1] = l;
+    }
+  }
+  __syncthreads();
+  for (int h = wave; h < REP; h += kAttnThreads / 64) {
+    float a0 = 0.f, a1 = 0.f;
+#pragma unroll
+    for (int i = 0; i < CHUNK; ++i) {                  // probabilities past kv_len are zero, their values were not loaded
+      const float p = sc[h][i];
+      a0 = __builtin_fmaf(p, vv0[i], a0);
+      if constexpr (D == 128) a1 = __builtin_fmaf(p, vv1[i], a1);
+    }
+    if constexpr (D == 128) *(v2f*)(out + h * (D + 2) + 2 * lane) = v2f{a0, a1};
+    else out[h * (D + 2) + lane] = a0;
+  }
+}
+
+// one workgroup of four waves per (sequence, query head): the chunks' partials -> fp16 output.  Every wave reads all
+// maxima and sums (lane s: chunk s, 64 chunks per pass; two wave reductions) and accumulates the weighted values of
+// every fourth chunk with the chunk's weight read from its lane; the four waves' sums meet in LDS.
+template <int D>
+__global__ __launch_bounds__(256) void decode_attention_combine_kernel(const float* __restrict__ partials,
+                                                                       __half* __restrict__ out, uint32_t rep,
+                                                                       uint32_t splits) {
+  __shared__ float acc[4][2][64];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const uint32_t bhq = blockIdx.x;                     // b * Hq + hq
+  const uint32_t bh = bhq / rep, h = bhq % rep;
+  const float* base = partials + (size_t)bh * splits * (rep * (D + 2)) + h * (D + 2);
+  const size_t stride = (size_t)rep * (D + 2);
+  float m = -INFINITY;
+  for (uint32_t s0 = 0; s0 < splits; s0 += 64)
+    if (s0 + lane < splits) m = __builtin_fmaxf(m, base[(s0 + lane) * stride + D]);
+  m = wave_max(m);
+  float l = 0.f, a0 = 0.f, a1 = 0.f;
+  for (uint32_t s0 = 0; s0 < splits; s0 += 64) {
+    float w = 0.f;
+    if (s0 + lane < splits) {
+      const float ms = base[(s0 + lane) * stride + D];
+      w = ms == -INFINITY ? 0.f : __expf(ms - m);
+      l = __builtin_fmaf(w, base[(s0 + lane) * stride + D + 1], l);
+    }
+    const uint32_t n = min(64u, splits - s0);
+#pragma unroll 4
+    for (uint32_t i = wave; i < n; i += 4) {
+      const float wi = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(w), (int)i));
+      if constexpr (D == 128) {
+        const v2f v = *(const v2f*)(base + (s0 + i) * stride + 2 * lane);
+        a0 = __builtin_fmaf(wi, v[0], a0);
+        a1 = __builtin_fmaf(wi, v[1], a1);
+      } else {
+        a0 = __builtin_fmaf(wi, base[(s0 + i) * stride + lane], a0);
+      }
+    }
+  }
+  l = wave_sum(l);
+  acc[wave][0][lane] = a0;
+  acc[wave][1][lane] = a1;
+  __syncthreads();
+  if (wave != 0) return;
+  a0 = (acc[0][0][lane] + acc[1][0][lane]) + (acc[2][0][lane] + acc[3][0][lane]);
+  a1 = (acc[0][1][lane] + acc[1][1][lane]) + (acc[2][1][lane] + acc[3][1][lane]);
+  const float inv = l > 0.f ? 1.0f / l : 0.f;
+  if constexpr (D == 128) {
+    const h2 r = {(_Float16)(a0 * inv), (_Float16)(a1 * inv)};
+    *(h2*)(out + (size_t)bhq * D + 2 * lane) = r;
+  } else {
+    out[(size_t)bhq * D + lane] = __float2half(a0 * inv);
+  }
+}
+
+constexpr int kChunk = 64;
+
+template <int D, int REP>
+int launch_attention(const __half* q, const __half* k, const __half* v, __half* out, float* partials, uint32_t B,
+                     uint32_t Hkv, uint32_t kv_len, uint32_t max_len, float scale, hipStream_t stream) {
+  const uint32_t splits = (kv_len + kChunk - 1) / kChunk;
+  hipLaunchKernelGGL((decode_attention_partial_kernel<D, REP, kChunk>), dim3(B * Hkv * splits), dim3(kAttnThreads), 0, stream,
+                     q, k, v, partials, Hkv, kv_len, max_len, splits, scale);
+  if (int rc = check_launch("decode_attention (partials)")) return rc;
+  hipLaunchKernelGGL((decode_attention_combine_kernel<D>), dim3(B * Hkv * REP), dim3(256), 0, stream, partials, out,
+                     (uint32_t)REP, splits);
+  return check_launch("decode_attention (combine)");
+}
+
+}  // namespace
+}  // namespace flh
+
+using namespace flh;
+
+extern "C" size_t flh_decode_attention_workspace_bytes(uint32_t B, uint32_t Hq, uint32_t head_dim, uint32_t kv_len) {
+  const size_t splits = ((size_t)kv_len + kChunk - 1) / kChunk;
+  return (size_t)B * Hq * splits * (head_dim + 2) * sizeof(float);
+}
+
+extern "C" int flh_decode_attention_f16(const flh_half* q, const flh_half* k_cache, const flh_half* v_cache, flh_half* out,
+                                        uint32_t B, uint32_t Hq, uint32_t Hkv, uint32_t head_dim, uint32_t kv_len,
+                                        uint32_t max_len, float scale, void* workspace, size_t workspace_bytes,
+                                        void* stream) {
+  if (!q || !k_cache || !v_cache || !out) return fail(FLH_EINVAL, "decode_attention: null pointer");
+  if (misaligned16(q, k_cache, v_cache, out)) return fail(FLH_EINVAL, "decode_attention: tensors must be 16-byte aligned");
+  if (head_dim != 128 && head_dim != 64) return fail(FLH_EINVAL, "decode_attention: head_dim (%u) must be 64 or 128", head_dim);
+  if (Hkv == 0 || Hq % Hkv) return fail(FLH_EINVAL, "decode_attention: %u query heads do not divide over %u key / value heads", Hq, Hkv);
+  const uint32_t rep = Hq / Hkv;
+  if (rep != 1 && rep != 2 && rep != 4 && rep != 8)
+    return fail(FLH_EINVAL, "decode_attention: %u query heads per key / value head (1, 2, 4 or 8 supported)", rep);
+  if (kv_len == 0 || kv_len > max_len) return fail(FLH_EINVAL, "decode_attention: kv_len (%u) must be in 1 .. max_len (%u)", kv_len, max_len);
+  if (B == 0) return FLH_OK;
+  const size_t need = flh_decode_attention_workspace_bytes(B, Hq, head_dim, kv_len);
+  if (!workspace || ((uintptr_t)workspace & 15)) return fail(FLH_EINVAL, "decode_attention: a 16-byte aligned workspace is required");
+  if (workspace_bytes < need)
+    return fail(FLH_EINVAL, "decode_attention: the workspace has %zu bytes, this call needs %zu", workspace_bytes, need);
+  if ((uint64_t)B * Hkv * ((kv_len + kChunk - 1) / kChunk) > 0x7FFFFFFFull) return fail(FLH_EINVAL, "decode_attention: too many chunks");
+  const __half *qh = (const __half*)q, *kh = (const __half*)k_cache, *vh = (const __half*)v_cache;
+  __half* oh = (__half*)out;
+  float* ws = (float*)workspace;
+  hipStream_t st = (hipStream_t)stream;
+#define FLH_ATTN(D, R) return launch_attention<D, R>(qh, kh, vh, oh, ws, B, Hkv, kv_len, max_len, scale, st)
+  if (head_dim == 128) {
+    switch (rep) {
+      case 1: FLH_ATTN(128, 1);
+      case 2: FLH_ATTN(128, 2);
+      case 4: FLH_ATTN(128, 4);
+      default: FLH_ATTN(128, 8);
+    }
+  }
+  switch (rep) {
+    case 1: FLH_ATTN(64, 1);
+    case 2: FLH_ATTN(64, 2);
+    case 4: FLH_ATTN(64, 4);
+    default: FLH_ATTN(64, 8);
+  }
+#undef FLH_ATTN
+}

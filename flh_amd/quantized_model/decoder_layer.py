@@ -77,11 +77,16 @@ class StaticKVCache:
     takes as `kv_cache`: new keys / values are written in place at `positions` (a device index tensor, so a captured
     graph can be replayed for other positions by overwriting it) and attention reads the first `kv_len` slots."""
 
-    def __init__(self, layers, batch, kv_heads, max_len, head_dim, device, dtype=torch.float16):
+    def __init__(self, layers, batch, kv_heads, max_len, head_dim, device, dtype=torch.float16, q_heads=None):
         self.keys = [torch.zeros(batch, kv_heads, max_len, head_dim, dtype=dtype, device=device) for _ in range(layers)]
         self.values = [torch.zeros_like(k) for k in self.keys]
         self.max_len = max_len
         self.kv_len = 0
+        # the decode-attention kernel's scratch (partial results of the chunks), shared by the layers: they run in
+        # order on one stream.  Owned here so that a captured graph finds it allocated.
+        q_heads = q_heads or kv_heads * 8
+        self.attention_workspace = torch.empty(batch * q_heads * ((max_len + 63) // 64) * (head_dim + 2) * 4,
+                                               dtype=torch.uint8, device=device)
 
     class _Layer:
         def __init__(self, owner, index):
@@ -94,6 +99,9 @@ class StaticKVCache:
             _ops().rope_kv_cache_(q, k, v, cos, sin, positions, keys, values)
             n = self.owner.kv_len
             return keys[:, :, :n], values[:, :, :n]
+
+        def tensors(self):
+            return self.owner.keys[self.index], self.owner.values[self.index]
 
     def layer(self, index):
         return StaticKVCache._Layer(self, index)
@@ -230,13 +238,20 @@ class W4A4DecoderLayer(torch.nn.Module):
         qs, ks, vs = self._project([self.q_proj, self.k_proj, self.v_proj], q, s, z)
         self._tap("q_proj", qs), self._tap("k_proj", ks), self._tap("v_proj", vs)
         static = isinstance(kv_cache, StaticKVCache._Layer)
+        out = None
         if static:
             # rotary embedding of q (in place) and k, and the new keys / values into their cache slots: one launch
             qs = qs.view(b, t, self.num_heads, self.head_dim)
             ks, vs = kv_cache.rope_and_update(qs, ks.view(b, t, self.num_kv_heads, self.head_dim),
                                               vs.view(b, t, self.num_kv_heads, self.head_dim), cos, sin, positions)
-            qs = qs.transpose(1, 2)
             cache = kv_cache
+            if t == 1 and self.head_dim in (64, 128) and self.num_heads // self.num_kv_heads in (1, 2, 4, 8):
+                # one new token against the cache: the chunked decode-attention kernel (two launches)
+                keys, values = kv_cache.tensors()
+                out = _ops().decode_attention(qs.view(b, self.num_heads, self.head_dim), keys, values, ks.size(2),
+                                              workspace=kv_cache.owner.attention_workspace)
+                out = out.view(b, 1, self.hidden_size)
+            qs = qs.transpose(1, 2)
         else:
             qs = qs.view(b, t, self.num_heads, self.head_dim).transpose(1, 2)
             ks = ks.view(b, t, self.num_kv_heads, self.head_dim).transpose(1, 2)
@@ -248,14 +263,15 @@ class W4A4DecoderLayer(torch.nn.Module):
             cache = (ks, vs)
         gqa = self.num_heads != self.num_kv_heads
         past = ks.size(2) - t
-        if t == 1 and past > 0:
-            out = _decode_attention(qs, ks, vs)           # one new token sees every cached position
-        elif past == 0:
-            out = torch.nn.functional.scaled_dot_product_attention(qs, ks, vs, is_causal=t > 1, enable_gqa=gqa)
-        else:
-            mask = torch.ones(t, past + t, dtype=torch.bool, device=x.device).tril(diagonal=past)
-            out = torch.nn.functional.scaled_dot_product_attention(qs, ks, vs, attn_mask=mask, enable_gqa=gqa)
-        out = out.transpose(1, 2).reshape(b, t, self.hidden_size).contiguous()
+        if out is None:
+            if t == 1 and past > 0:
+                out = _decode_attention(qs, ks, vs)           # one new token sees every cached position
+            elif past == 0:
+                out = torch.nn.functional.scaled_dot_product_attention(qs, ks, vs, is_causal=t > 1, enable_gqa=gqa)
+            else:
+                mask = torch.ones(t, past + t, dtype=torch.bool, device=x.device).tril(diagonal=past)
+                out = torch.nn.functional.scaled_dot_product_attention(qs, ks, vs, attn_mask=mask, enable_gqa=gqa)
+            out = out.transpose(1, 2).reshape(b, t, self.hidden_size).contiguous()
         if (self.activation == "token" and self.fused and self.record is None and b * t <= 2
                 and self.hidden_size == 4096):
             # decode: the quantiser runs inside the GEMM's own launch (same bits as the two launches)

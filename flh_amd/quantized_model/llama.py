@@ -82,7 +82,7 @@ class W4A4LlamaModel(torch.nn.Module):
     def new_cache(self, batch, max_len):
         s = self.shape
         dev = self.embed_tokens.weight.device
-        return StaticKVCache(s.num_layers, batch, s.num_kv_heads, max_len, s.head_dim, dev)
+        return StaticKVCache(s.num_layers, batch, s.num_kv_heads, max_len, s.head_dim, dev, q_heads=s.num_heads)
 
     def embed(self, input_ids):
         x = self.embed_tokens(input_ids)

@@ -249,6 +249,20 @@ int flh_rope_kv_cache_f16(flh_half* q, const flh_half* k, const flh_half* v, con
                           const int64_t* positions, flh_half* k_cache, flh_half* v_cache, uint32_t B, uint32_t T,
                           uint32_t Hq, uint32_t Hkv, uint32_t head_dim, uint32_t max_len, void* stream);
 
+/* Attention of ONE new token per sequence over the cache that flh_rope_kv_cache_f16 fills (the decode step), grouped
+ * queries included:  out[b, h] = softmax(q[b, h] . K[b, h / rep]^T * scale) V[b, h / rep]  over cache slots [0, kv_len),
+ * rep = Hq / Hkv in {1, 2, 4, 8}, head_dim 64 or 128; scores, probabilities and sums in float32, fp16 in and out.
+ *   q, out [B, Hq, d];  k_cache, v_cache [B, Hkv, max_len, d].
+ * Stands where the reference's attention calls the flash-attn package on the cached keys / values
+ * (flh/quantized_model/modeling_llama.py:449-460).  The cached positions are split into chunks of 64 that run in
+ * parallel; their partial results meet in `workspace` (device memory, 16-byte aligned, at least
+ * flh_decode_attention_workspace_bytes(B, Hq, d, kv_len) bytes, contents irrelevant before and after; launches that
+ * share a workspace must not overlap, i.e. one workspace per stream).  Two launches on `stream`. */
+size_t flh_decode_attention_workspace_bytes(uint32_t B, uint32_t Hq, uint32_t head_dim, uint32_t kv_len);
+int flh_decode_attention_f16(const flh_half* q, const flh_half* k_cache, const flh_half* v_cache, flh_half* out,
+                             uint32_t B, uint32_t Hq, uint32_t Hkv, uint32_t head_dim, uint32_t kv_len, uint32_t max_len,
+                             float scale, void* workspace, size_t workspace_bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif
