@@ -224,3 +224,46 @@ extern "C" int flh_decode_attention_f16(const flh_half* q, const flh_half* k_cac
   }
 #undef FLH_ATTN
 }
+
+// ---- the same for callers that cannot allocate ---------------------------------------------------------------------
+// The partials live in a static device array of a fixed size instead of a caller's workspace.  Every device the library
+// runs on holds its own copy of the array until the process ends; the address of the current device's copy is looked
+// up once per device.  Calls on one device share that array: calls that overlap in time (different streams) race.
+constexpr size_t kScratchBytes = 16u << 20;            // 16 MiB: e.g. 31 sequences x 32 query heads x 2048 positions, d = 128
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::atomic<void*> g_scratch_ptr[kMaxDevices];         // per device: where that device's copy of `scratch` lives
+
+int scratch_of_current_device(void** out) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return fail(FLH_EDEVICE, "decode_attention: no current HIP device");
+  if (dev < 0 || dev >= kMaxDevices) return fail(FLH_EDEVICE, "decode_attention: device index %d out of range", dev);
+  void* ptr = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (!ptr) {
+    const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));   // of the current device
+    if (e != hipSuccess || !ptr)
+      return fail(FLH_ELAUNCH, "decode_attention: cannot locate the static scratch array: %s", hipGetErrorString(e));
+    g_scratch_ptr[dev].store(ptr, std::memory_order_release);
+  }
+  *out = ptr;
+  return FLH_OK;
+}
+}  // namespace
+
+extern "C" size_t flh_decode_attention_static_scratch_bytes(void) { return kScratchBytes; }
+
+extern "C" int flh_decode_attention_f16_static(const flh_half* q, const flh_half* k_cache, const flh_half* v_cache,
+                                               flh_half* out, uint32_t B, uint32_t Hq, uint32_t Hkv, uint32_t head_dim,
+                                               uint32_t kv_len, uint32_t max_len, float scale, void* stream) {
+  const size_t need = flh_decode_attention_workspace_bytes(B, Hq, head_dim, kv_len);
+  if (need > kScratchBytes)
+    return fail(FLH_EINVAL, "decode_attention (static scratch): this call needs %zu bytes of scratch, the static array has "
+                "%zu; use flh_decode_attention_f16 with a workspace", need, kScratchBytes);
+  void* ptr = nullptr;
+  if (int e = scratch_of_current_device(&ptr)) return e;
+  // every chunk's partial is written before the combine kernel reads it: nothing has to start at zero
+  return flh_decode_attention_f16(q, k_cache, v_cache, out, B, Hq, Hkv, head_dim, kv_len, max_len, scale, ptr,
+                                  kScratchBytes, stream);
+}

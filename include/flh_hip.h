@@ -263,6 +263,18 @@ int flh_decode_attention_f16(const flh_half* q, const flh_half* k_cache, const f
                              uint32_t B, uint32_t Hq, uint32_t Hkv, uint32_t head_dim, uint32_t kv_len, uint32_t max_len,
                              float scale, void* workspace, size_t workspace_bytes, void* stream);
 
+/* flh_decode_attention_f16 for callers that cannot allocate device memory and have no workspace to hand over -- code
+ * under stream capture, tight serving loops, harnesses that forbid allocation.  No counterpart in the reference.  It
+ * allocates nothing: the partial results go to a static device array of flh_decode_attention_static_scratch_bytes()
+ * (16 MiB) that every device the library runs on holds until the process ends.  A call that needs more
+ * (B * Hq * ceil(kv_len / 64) * (head_dim + 2) * 4 bytes) is rejected with FLH_EINVAL.  All calls on one device share the
+ * array: calls that overlap in time (different streams) race; calls on one stream do not.  Same results, bit for bit,
+ * as flh_decode_attention_f16. */
+size_t flh_decode_attention_static_scratch_bytes(void);
+int flh_decode_attention_f16_static(const flh_half* q, const flh_half* k_cache, const flh_half* v_cache, flh_half* out,
+                                    uint32_t B, uint32_t Hq, uint32_t Hkv, uint32_t head_dim, uint32_t kv_len,
+                                    uint32_t max_len, float scale, void* stream);
+
 #ifdef __cplusplus
 }
 #endif
