@@ -491,6 +491,40 @@ def silu_mul_and_quantize_i4_gs(gate, up, group_size, hadamard=False, *, scale_m
     return [q, s]
 
 
+SILU_ROTATE_MAX_ROWS = 256
+
+
+def silu_mul(gate, up):
+    """fp16(fp16(silu(gate)) * up) elementwise in one launch (fp16 tensors of one shape, element count a multiple of 8)."""
+    _check(gate.is_cuda and up.is_cuda and gate.device == up.device, "Input tensors must be on CUDA")
+    _check(gate.dtype == torch.float16 and up.dtype == torch.float16, "Input tensors must be float16 (half)")
+    _check(gate.shape == up.shape and gate.is_contiguous() and up.is_contiguous(),
+           "gate and up must be contiguous tensors of one shape")
+    _check(gate.numel() % 8 == 0, "element count must be a multiple of 8")
+    out = torch.empty_like(gate)
+    if gate.numel():
+        _run("flh_silu_mul_f16", gate.device, gate.data_ptr(), up.data_ptr(), out.data_ptr(), gate.numel(), _stream(gate))
+    return out
+
+
+def silu_mul_rotate_and_quantize_i4(gate, up):
+    """Decode-sized batches: rotate_and_quantize_i4(silu(gate) * up, hadamard="fast") in one launch that never stores the
+    product: gate, up [M, K] fp16 with K = 11008 or 14336, M <= 256 -> (q [M, K/2] u8, scales [M, 1] fp16)."""
+    _check(gate.is_cuda and up.is_cuda and gate.device == up.device, "Input tensors must be on CUDA")
+    _check(gate.dtype == torch.float16 and up.dtype == torch.float16, "Input tensors must be float16 (half)")
+    _check(gate.dim() == 2 and gate.shape == up.shape and gate.is_contiguous() and up.is_contiguous(),
+           "gate and up must be contiguous 2D tensors of one shape")
+    M, K = gate.shape
+    _check(K in (11008, 14336), "Last dimension must be 11008 or 14336")
+    _check(M <= SILU_ROTATE_MAX_ROWS, "at most 256 rows")
+    q = torch.empty((M, K // 2), dtype=torch.uint8, device=gate.device)
+    s = torch.empty((M, 1), dtype=torch.float16, device=gate.device)
+    if M:
+        _run("flh_silu_mul_rotate_quant_i4", gate.device, gate.data_ptr(), up.data_ptr(), q.data_ptr(), s.data_ptr(), M, K,
+             _stream(gate))
+    return q, s
+
+
 def rmsnorm_and_quantize_i4_gs(x, weight, eps, group_size, hadamard=False, *, scale_mul=1.0):
     """RMSNorm (flh/nn/normalization.py:12-20) + group quantiser in one launch: x [..., K] fp16,
     weight [K] fp16 or None -> [q [..., K/2] u8, scales [..., K/group_size] fp16]."""
@@ -534,6 +568,29 @@ def rmsnorm_rotate_and_quantize_i4(x, weight, eps, hadamard=True, clip_ratio=1.0
              float(eps), q.data_ptr(), s.data_ptr(), y.data_ptr() if y is not None else None, M, K,
              FLH_HAD_F32 if hadamard else FLH_HAD_NONE, float(clip_ratio), _stream(x))
     return (q, s, y) if return_rotated else (q, s)
+
+
+def add_rmsnorm_rotate_and_quantize_i4(x, add, weight, eps, hadamard=True, clip_ratio=1.0):
+    """The residual addition in front of rmsnorm_rotate_and_quantize_i4, in the same launch: x, add [M, K] fp16 ->
+    (x + add [M, K] fp16, q [M, K/2] u8, scales [M, 1] fp16), q and scales those of
+    rmsnorm_rotate_and_quantize_i4(x + add, weight, eps, hadamard, clip_ratio)."""
+    _check(x.is_cuda and add.is_cuda and x.device == add.device, "Input tensors must be on CUDA")
+    _check(x.dtype == torch.float16 and add.dtype == torch.float16, "Input tensors must be float16 (half)")
+    _check(x.dim() == 2 and x.shape == add.shape and x.is_contiguous() and add.is_contiguous(),
+           "x and add must be contiguous 2D tensors of one shape")
+    M, K = x.shape
+    _check(K in (512, 1024, 2048, 4096, 8192), "Last dimension must be 512, 1024, 2048, 4096 or 8192")
+    if weight is not None:
+        _check(weight.is_cuda and weight.dtype == torch.float16 and weight.is_contiguous() and weight.numel() == K,
+               "weight must be a contiguous float16 CUDA tensor of K values")
+    total = torch.empty_like(x)
+    q = torch.empty((M, K // 2), dtype=torch.uint8, device=x.device)
+    s = torch.empty((M, 1), dtype=torch.float16, device=x.device)
+    if M:
+        _run("flh_add_rmsnorm_rotate_quant_i4", x.device, x.data_ptr(), add.data_ptr(), total.data_ptr(),
+             weight.data_ptr() if weight is not None else None, float(eps), q.data_ptr(), s.data_ptr(), M, K,
+             FLH_HAD_F32 if hadamard else FLH_HAD_NONE, float(clip_ratio), _stream(x))
+    return total, q, s
 
 
 def rotate_and_quantize_i4(x, hadamard=True, had_group=0, scale_group=0, clip_ratio=1.0, return_rotated=False):

@@ -297,12 +297,19 @@ __device__ __forceinline__ v2i quantise_half_block(const unsigned (&y)[8], float
 // loads, 16-byte chunks XOR-swizzled by the row so that the tile reads are free of bank conflicts), instead of
 // every wave waiting for its X tiles from memory three at a time (in-kernel timestamps for one row of 14336: the
 // main loop took 13 k clocks of a 23 k clock kernel, almost all of it waiting for those tiles).
-template <int DT, bool SPLIT>
+//
+// SILU (short batches only): the row is the SwiGLU product fp16(fp16(silu(gate)) * up) of two input rows, x = gate and
+// x2 = up -- what the reference's MLP hands to the quantiser of down_proj (flh/quantized_model/modeling_llama.py:522-526).
+// Both rows are staged in LDS the same way and combined in place before the first tile is read, so the product never
+// goes to memory.
+template <int DT, bool SPLIT, bool SILU = false>
 __global__ __launch_bounds__(512) void rotate_quant_mfma_dense_kernel(const __half* __restrict__ x,
                                                                        uint8_t* __restrict__ q,
                                                                        __half* __restrict__ scales,
                                                                        const h8* __restrict__ table, uint32_t M,
-                                                                       float inv_norm, float clip) {
+                                                                       float inv_norm, float clip,
+                                                                       const __half* __restrict__ x2 = nullptr) {
+  static_assert(!SILU || SPLIT, "the SwiGLU prologue works on the row staged in LDS");
   constexpr int D = DenseFactor<DT>::D, K = D * 64, NFRAG = 2 * DT * DT;
   extern __shared__ __align__(1024) h8 mfrag[];        // [kb][s][nt][lane], then the maxima
   float* red = (float*)(mfrag + NFRAG * 64);           // [parity][row slot][mt]
@@ -363,6 +370,8 @@ __global__ __launch_bounds__(512) void rotate_quant_mfma_dense_kernel(const __ha
     for (int i = wave; i < DT * 4; i += 8) {
       const int j = 8 * i + (lane >> 3), c = (lane & 7) ^ (j & 7);
       load_to_lds16(xr + (j < D ? j : D - 1) * 64 + c * 8, xs0 + i * 1024);
+      if constexpr (SILU)                              // the up row behind the gate row, same slot order
+        load_to_lds16(x2 + (xr - x) + (j < D ? j : D - 1) * 64 + c * 8, xs0 + DT * 4096 + i * 1024);
     }
   } else if (base0 < M) {
 #pragma unroll
@@ -376,6 +385,18 @@ __global__ __launch_bounds__(512) void rotate_quant_mfma_dense_kernel(const __ha
       load_to_lds16(table + f * 64 + lane, lds0 + f * 1024);
     }
     wait_vmcnt<0>();
+    __syncthreads();
+  }
+  if constexpr (SILU) {
+    h8* g8 = (h8*)xs;
+    const h8* u8 = (const h8*)(xs + DT * 4096);
+    for (int i = threadIdx.x; i < DT * 256; i += 512) {
+      const h8 g = g8[i], u = u8[i];
+      h8 o;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) o[e] = silu_mul_f16(g[e], u[e]);
+      g8[i] = o;
+    }
     __syncthreads();
   }
   if constexpr (SPLIT) {
@@ -512,6 +533,25 @@ int dense_table(const h8** out) {
   return FLH_OK;
 }
 
+// the SwiGLU product of two rows in front of the rotation (short batches: one row per workgroup)
+template <int DT>
+int launch_dense_silu(const __half* gate, const __half* up, uint8_t* q, __half* scales, uint32_t M, hipStream_t stream) {
+  constexpr int NFRAG = 2 * DT * DT;
+  constexpr int K = DenseFactor<DT>::D * 64;
+  const h8* table = nullptr;
+  if (int rc = dense_table<DT>(&table)) return rc;
+  const size_t smem = (size_t)NFRAG * 1024 + 64 + 2 * (size_t)DT * 4096;   // factor fragments, maxima, gate row, up row
+  auto kern = rotate_quant_mfma_dense_kernel<DT, true, true>;
+  static std::atomic<bool> attr{false};
+  if (!attr.load(std::memory_order_acquire)) {
+    if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess)
+      return fail(FLH_ELAUNCH, "silu_mul_rotate_quant: cannot reserve %zu bytes of LDS", smem);
+    attr.store(true, std::memory_order_release);
+  }
+  hipLaunchKernelGGL(kern, dim3(M), dim3(512), smem, stream, gate, q, scales, table, M, 1.0f / sqrtf((float)K), 1.0f, up);
+  return check_launch("silu_mul_rotate_quant");
+}
+
 template <int DT>
 int launch_dense(const __half* x, uint8_t* q, __half* scales, uint32_t M, float clip, hipStream_t stream) {
   constexpr int NFRAG = 2 * DT * DT;
@@ -532,7 +572,7 @@ int launch_dense(const __half* x, uint8_t* q, __half* scales, uint32_t M, float 
   }
   const unsigned blocks = split ? M : ((M + 3) / 4 < 256u ? (M + 3) / 4 : 256u);
   hipLaunchKernelGGL(kern, dim3(blocks), dim3(kThreadsDense), smem, stream, x, q, scales, table, M,
-                     1.0f / sqrtf((float)K), clip);
+                     1.0f / sqrtf((float)K), clip, (const __half*)nullptr);
   return check_launch("rotate_quant_mfma_dense");
 }
 
@@ -545,6 +585,14 @@ int rotate_quant_mfma_init() {
   const h8* t = nullptr;
   if (int rc = dense_table<6>(&t)) return rc;
   return dense_table<7>(&t);
+}
+
+// launcher used by flh_silu_mul_rotate_quant_i4 (fwht_quant.hip): K = 11008 / 14336, at most kSiluRotateMaxRows rows
+int launch_silu_mul_rotate_quant_mfma(const __half* gate, const __half* up, uint8_t* q, __half* scales, uint32_t M,
+                                      uint32_t K, hipStream_t stream) {
+  if (K == 11008) return launch_dense_silu<6>(gate, up, q, scales, M, stream);
+  if (K == 14336) return launch_dense_silu<7>(gate, up, q, scales, M, stream);
+  return fail(FLH_EINVAL, "silu_mul_rotate_quant: K = %u is not supported (11008 or 14336)", K);
 }
 
 // launcher used by flh_rotate_quant_i4 (fwht_quant.hip)

@@ -255,6 +255,18 @@ __global__ __launch_bounds__(256) void silu_mul_group_kernel(const __half* __res
   group_finish<G>(v, lir, valid, row, q, scales, scale_mul);
 }
 
+// the SwiGLU product alone, eight values per thread
+__global__ __launch_bounds__(256) void silu_mul_kernel(const __half* __restrict__ gate, const __half* __restrict__ up,
+                                                       __half* __restrict__ out, uint64_t chunks) {
+  const uint64_t i = (uint64_t)blockIdx.x * 256u + threadIdx.x;
+  if (i >= chunks) return;
+  const h8 g = *(const h8*)(gate + i * 8), u = *(const h8*)(up + i * 8);
+  h8 o;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) o[e] = silu_mul_f16(g[e], u[e]);
+  *(h8*)(out + i * 8) = o;
+}
+
 // RMSNorm in front of the group kernel, one workgroup per token row of K = 8 * chunks values (K <= 16384):
 // y = fp16( float(x) * rsqrt(sum(x^2) / K + eps) [* float(weight)] ) with the statistics in float32
 // (flh/nn/normalization.py:12-20), then transform + quantise per group of G as group_kernel<G, HAD, true>.
@@ -321,12 +333,15 @@ __global__ __launch_bounds__(256) void rotate_quant_wave_kernel(const __half* __
                                                                 __half* __restrict__ scales,
                                                                 __half* __restrict__ y_out, uint32_t M, float norm,
                                                                 float clip, const __half* __restrict__ rms_weight = nullptr,
-                                                                float rms_eps = 0.f) {
+                                                                float rms_eps = 0.f, const __half* add = nullptr,
+                                                                __half* sum_out = nullptr) {
   constexpr int K = 512 * J;
   const uint32_t row = blockIdx.x * 4u + (threadIdx.x >> 6);
   if (row >= M) return;  // wave-uniform
   rotate_quant_row<J, HAD, EXACT_NORM, RMS>(x + (size_t)row * K, q + (size_t)row * (K / 2), scales + row,
-                                            y_out ? y_out + (size_t)row * K : nullptr, norm, clip, rms_weight, rms_eps);
+                                            y_out ? y_out + (size_t)row * K : nullptr, norm, clip, rms_weight, rms_eps,
+                                            add ? add + (size_t)row * K : nullptr,
+                                            add ? sum_out + (size_t)row * K : nullptr);
 }
 
 constexpr int kGenericThreads = 1024;      // one workgroup per compute unit (LDS): two waves per SIMD hide latencies
@@ -551,13 +566,15 @@ int launch_wave(const __half* x, uint8_t* q, __half* s, __half* y, uint32_t M, b
   const bool even = (lg % 2) == 0;
   const dim3 grid((M + 3) / 4), block(256);
   if (!had)
-    hipLaunchKernelGGL((rotate_quant_wave_kernel<J, false, true>), grid, block, 0, stream, x, q, s, y, M, 1.0f, clip);
+    hipLaunchKernelGGL((rotate_quant_wave_kernel<J, false, true>), grid, block, 0, stream, x, q, s, y, M, 1.0f, clip,
+                       (const __half*)nullptr, 0.f, (const __half*)nullptr, (__half*)nullptr);
   else if (even)
     hipLaunchKernelGGL((rotate_quant_wave_kernel<J, true, true>), grid, block, 0, stream, x, q, s, y, M,
-                       1.0f / (float)(1 << (lg / 2)), clip);
+                       1.0f / (float)(1 << (lg / 2)), clip, (const __half*)nullptr, 0.f, (const __half*)nullptr,
+                       (__half*)nullptr);
   else
     hipLaunchKernelGGL((rotate_quant_wave_kernel<J, true, false>), grid, block, 0, stream, x, q, s, y, M,
-                       sqrtf((float)K), clip);
+                       sqrtf((float)K), clip, (const __half*)nullptr, 0.f, (const __half*)nullptr, (__half*)nullptr);
   return check_launch("rotate_quant_wave");
 }
 
@@ -583,26 +600,40 @@ __global__ __launch_bounds__(512) void rmsnorm_rotate_quant_row8_kernel(const __
   const size_t row = blockIdx.x;
   rotate_quant_row_8waves<true>(x + row * 4096, stage, wave_max8, q + row * 2048, scales + row, norm, wave, weight, eps);
 }
+// ... and with the residual addition in front of that (flh_add_rmsnorm_rotate_quant_i4)
+__global__ __launch_bounds__(512) void add_rmsnorm_rotate_quant_row8_kernel(const __half* __restrict__ x,
+                                                                            const __half* __restrict__ add,
+                                                                            __half* __restrict__ sum_out,
+                                                                            const __half* __restrict__ weight, float eps,
+                                                                            uint8_t* __restrict__ q,
+                                                                            __half* __restrict__ scales, float norm) {
+  __shared__ float stage[8 * 8 * 64];
+  __shared__ float wave_max8[8];
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const size_t row = blockIdx.x;
+  rotate_quant_row_8waves<true, true>(x + row * 4096, stage, wave_max8, q + row * 2048, scales + row, norm, wave, weight,
+                                      eps, add + row * 4096, sum_out + row * 4096);
+}
 // measured per launch inside a replayed graph: 2.7 against 4.4 us for one row, 3.2 against 4.9 us for 256 rows,
 // 3.9 against 5.0 us for 512; from 1024 rows on the wave-per-row kernel is the faster one
 constexpr uint32_t kRow8MaxRows = 512;
 
 template <int J>
 int launch_wave_rms(const __half* x, const __half* w, float eps, uint8_t* q, __half* s, __half* y, uint32_t M, bool had,
-                    float clip, hipStream_t stream) {
+                    float clip, hipStream_t stream, const __half* add = nullptr, __half* sum_out = nullptr) {
   constexpr int K = 512 * J;
   int lg = 0;
   while ((1 << lg) < K) ++lg;
   const dim3 grid((M + 3) / 4), block(256);
   if (!had)
     hipLaunchKernelGGL((rotate_quant_wave_kernel<J, false, true, true>), grid, block, 0, stream, x, q, s, y, M, 1.0f,
-                       clip, w, eps);
+                       clip, w, eps, add, sum_out);
   else if (lg % 2 == 0)
     hipLaunchKernelGGL((rotate_quant_wave_kernel<J, true, true, true>), grid, block, 0, stream, x, q, s, y, M,
-                       1.0f / (float)(1 << (lg / 2)), clip, w, eps);
+                       1.0f / (float)(1 << (lg / 2)), clip, w, eps, add, sum_out);
   else
     hipLaunchKernelGGL((rotate_quant_wave_kernel<J, true, false, true>), grid, block, 0, stream, x, q, s, y, M,
-                       sqrtf((float)K), clip, w, eps);
+                       sqrtf((float)K), clip, w, eps, add, sum_out);
   return check_launch("rmsnorm_rotate_quant_wave");
 }
 
@@ -663,6 +694,8 @@ int launch_rmsnorm(const __half* x, const __half* w, uint8_t* q, __half* s, uint
 int launch_rotate_quant_mfma(const __half* x, uint8_t* q, __half* scales, uint32_t M, uint32_t K, float clip,
                              hipStream_t stream);
 bool rotate_quant_mfma_supports(uint32_t K);
+int launch_silu_mul_rotate_quant_mfma(const __half* gate, const __half* up, uint8_t* q, __half* scales, uint32_t M,
+                                      uint32_t K, hipStream_t stream);
 
 }  // namespace flh
 
@@ -739,6 +772,63 @@ extern "C" int flh_rmsnorm_rotate_quant_i4(const flh_half* x, const flh_half* we
     case 8: return launch_wave_rms<8>(xh, wh, eps, q_packed, sh, yh, M, had, clip_ratio, st);
     default: return launch_wave_rms<16>(xh, wh, eps, q_packed, sh, yh, M, had, clip_ratio, st);
   }
+}
+
+extern "C" int flh_add_rmsnorm_rotate_quant_i4(const flh_half* x, const flh_half* add, flh_half* sum_out,
+                                               const flh_half* weight, float eps, uint8_t* q_packed, flh_half* scales,
+                                               uint32_t M, uint32_t K, int hadamard, float clip_ratio, void* stream) {
+  if (!x || !add || !sum_out || !q_packed || !scales) return fail(FLH_EINVAL, "add_rmsnorm_rotate_quant: null pointer");
+  if (misaligned16(x, add, sum_out) || misaligned16(q_packed))
+    return fail(FLH_EINVAL, "add_rmsnorm_rotate_quant: x, add, sum_out and q_packed must be 16-byte aligned");
+  if (weight && misaligned16(weight)) return fail(FLH_EINVAL, "add_rmsnorm_rotate_quant: weight must be 16-byte aligned");
+  if (!(clip_ratio > 0.f)) return fail(FLH_EINVAL, "add_rmsnorm_rotate_quant: clip_ratio must be positive");
+  if (!(eps >= 0.f)) return fail(FLH_EINVAL, "add_rmsnorm_rotate_quant: eps must not be negative");
+  if (hadamard != FLH_HAD_NONE && hadamard != FLH_HAD_F32)
+    return fail(FLH_EINVAL, "add_rmsnorm_rotate_quant: hadamard mode must be FLH_HAD_NONE or FLH_HAD_F32");
+  if (K % 512 || !is_pow2(K / 512) || K > 8192)
+    return fail(FLH_EINVAL, "add_rmsnorm_rotate_quant: K (%u) must be 512, 1024, 2048, 4096 or 8192", K);
+  if (M == 0) return FLH_OK;
+  const __half *xh = (const __half*)x, *ah = (const __half*)add, *wh = (const __half*)weight;
+  __half *sh = (__half*)scales, *oh = (__half*)sum_out;
+  const bool had = hadamard != FLH_HAD_NONE;
+  hipStream_t st = (hipStream_t)stream;
+  // (the eight-waves-per-row kernel lets other waves read x and add after one has stored its part of the sum)
+  if ((const void*)sum_out == (const void*)x || (const void*)sum_out == (const void*)add)
+    return fail(FLH_EINVAL, "add_rmsnorm_rotate_quant: sum_out must not be x or add");
+  if (had && K == 4096 && clip_ratio >= 1.0f && M <= kRow8MaxRows) {
+    hipLaunchKernelGGL(add_rmsnorm_rotate_quant_row8_kernel, dim3(M), dim3(512), 0, st, xh, ah, oh, wh, eps, q_packed, sh,
+                       1.0f / 64.0f);
+    return check_launch("add_rmsnorm_rotate_quant_row8");
+  }
+  switch (K / 512) {
+    case 1: return launch_wave_rms<1>(xh, wh, eps, q_packed, sh, nullptr, M, had, clip_ratio, st, ah, oh);
+    case 2: return launch_wave_rms<2>(xh, wh, eps, q_packed, sh, nullptr, M, had, clip_ratio, st, ah, oh);
+    case 4: return launch_wave_rms<4>(xh, wh, eps, q_packed, sh, nullptr, M, had, clip_ratio, st, ah, oh);
+    case 8: return launch_wave_rms<8>(xh, wh, eps, q_packed, sh, nullptr, M, had, clip_ratio, st, ah, oh);
+    default: return launch_wave_rms<16>(xh, wh, eps, q_packed, sh, nullptr, M, had, clip_ratio, st, ah, oh);
+  }
+}
+
+extern "C" int flh_silu_mul_f16(const flh_half* gate, const flh_half* up, flh_half* out, uint64_t n, void* stream) {
+  if (!gate || !up || !out) return fail(FLH_EINVAL, "silu_mul: null pointer");
+  if (misaligned16(gate, up, out)) return fail(FLH_EINVAL, "silu_mul: gate, up and out must be 16-byte aligned");
+  if (n % 8) return fail(FLH_EINVAL, "silu_mul: the element count (%llu) must be a multiple of 8", (unsigned long long)n);
+  if (n / 8 > 0x7fffffffull * 256) return fail(FLH_EINVAL, "silu_mul: too many elements");
+  if (n == 0) return FLH_OK;
+  hipLaunchKernelGGL(silu_mul_kernel, dim3((unsigned)((n / 8 + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
+                     (const __half*)gate, (const __half*)up, (__half*)out, n / 8);
+  return check_launch("silu_mul_kernel");
+}
+
+extern "C" int flh_silu_mul_rotate_quant_i4(const flh_half* gate, const flh_half* up, uint8_t* q_packed, flh_half* scales,
+                                            uint32_t M, uint32_t K, void* stream) {
+  if (!gate || !up || !q_packed || !scales) return fail(FLH_EINVAL, "silu_mul_rotate_quant: null pointer");
+  if (misaligned16(gate, up, q_packed)) return fail(FLH_EINVAL, "silu_mul_rotate_quant: gate, up and q_packed must be 16-byte aligned");
+  if (K != 11008 && K != 14336) return fail(FLH_EINVAL, "silu_mul_rotate_quant: K (%u) must be 11008 or 14336", K);
+  if (M > 256) return fail(FLH_EINVAL, "silu_mul_rotate_quant: at most 256 rows (%u given); longer batches take the gate / up GEMM that stores the product", M);
+  if (M == 0) return FLH_OK;
+  return launch_silu_mul_rotate_quant_mfma((const __half*)gate, (const __half*)up, q_packed, (__half*)scales, M, K,
+                                           (hipStream_t)stream);
 }
 
 extern "C" int flh_group_quant_f6(const flh_half* x, uint8_t* encoded, flh_half* scales, uint32_t M, uint32_t K,

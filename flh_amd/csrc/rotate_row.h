@@ -70,13 +70,31 @@ __device__ __forceinline__ void stage_swap(float (&v)[N]) {
   }
 }
 
+// eight fp16 additions (four packed pairs), each rounded once
+__device__ __forceinline__ v4i add_h8(v4i a, v4i b) {
+  v4i r;
+#pragma unroll
+  for (int d = 0; d < 4; ++d) {
+    const unsigned ua = (unsigned)a[d], ub = (unsigned)b[d];   // (scalar copies: a bit cast of a vector element miscompiles)
+    const h2 s2 = __builtin_bit_cast(h2, ua) + __builtin_bit_cast(h2, ub);
+    r[d] = (int)__builtin_bit_cast(unsigned, s2);
+  }
+  return r;
+}
+
 // RMS: the row is first normalised as flh/nn/normalization.py:12-20 does -- float32 sum of squares / K,
 // x * (1 / sqrt(. + eps)) [* weight] with every product rounded to float32, then fp16 -- and that fp16 row is
 // what the rotation and the quantiser see.
+//
+// add_row / sum_row (both or neither): the row is x + add in fp16 (one rounding per value, torch's fp16 addition), and
+// that sum is also stored to sum_row -- the residual stream of a decoder layer (modeling_llama.py:600-618:
+// hidden = residual + attention output; residual = hidden; hidden = norm(hidden)) without a launch of its own.
+// sum_row overlaps neither input.
 template <int J, bool HAD, bool EXACT_NORM, bool RMS = false>
 __device__ __forceinline__ void rotate_quant_row(const __half* __restrict__ x_row, uint8_t* q_row, __half* scale_dst,
                                                  __half* y_row, float norm, float clip,
-                                                 const __half* __restrict__ rms_weight = nullptr, float rms_eps = 0.f) {
+                                                 const __half* __restrict__ rms_weight = nullptr, float rms_eps = 0.f,
+                                                 const __half* add_row = nullptr, __half* sum_row = nullptr) {
   constexpr int K = 512 * J, N = 8 * J;
   const int lane = threadIdx.x & 63;
   const int c = lane_chunk(lane);
@@ -85,6 +103,12 @@ __device__ __forceinline__ void rotate_quant_row(const __half* __restrict__ x_ro
   v4i raw[J];
 #pragma unroll
   for (int j = 0; j < J; ++j) raw[j] = *(const v4i*)(xr + j * 512);
+  if (add_row) {                                       // wave-uniform
+#pragma unroll
+    for (int j = 0; j < J; ++j) raw[j] = add_h8(raw[j], *(const v4i*)(add_row + c * 8 + j * 512));
+#pragma unroll
+    for (int j = 0; j < J; ++j) *(v4i*)(sum_row + c * 8 + j * 512) = raw[j];
+  }
 
   if constexpr (RMS) {
     float ss = 0.f;
@@ -225,19 +249,27 @@ __device__ __forceinline__ void rotate_quant_row(const __half* __restrict__ x_ro
 // more (it is in the compute unit's cache by then) and sums the squares in exactly that routine's order -- per lane
 // over the eight 512-value segments, then the fixed tree over the lanes -- so that the statistics, the normalised
 // fp16 row and therefore the codes are bit-identical to the wave-per-row kernel's, without a pass over the waves.
-template <bool RMS = false>
+// ADD: the row is x + add_row (fp16), stored to sum_row as well, as in rotate_quant_row.  Every wave forms the whole sum
+// for the statistics and stores only its own segment (the other waves still read x_row and add_row meanwhile).
+template <bool RMS = false, bool ADD = false>
 __device__ __forceinline__ void rotate_quant_row_8waves(const __half* __restrict__ x_row, float* stage, float* wave_max8,
                                                         uint8_t* q_row, __half* scale_dst, float norm, int wave,
                                                         const __half* __restrict__ rms_weight = nullptr,
-                                                        float rms_eps = 0.f) {
+                                                        float rms_eps = 0.f, const __half* __restrict__ add_row = nullptr,
+                                                        __half* __restrict__ sum_row = nullptr) {
   const int lane = threadIdx.x & 63;
   const int c = lane_chunk(lane);
   v4i raw = *(const v4i*)(x_row + wave * 512 + c * 8);
+  if constexpr (ADD) {
+    raw = add_h8(raw, *(const v4i*)(add_row + wave * 512 + c * 8));
+    *(v4i*)(sum_row + wave * 512 + c * 8) = raw;
+  }
   if constexpr (RMS) {
     float ss = 0.f;
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
-      const v4i seg = *(const v4i*)(x_row + j * 512 + c * 8);
+      v4i seg = *(const v4i*)(x_row + j * 512 + c * 8);
+      if constexpr (ADD) seg = add_h8(seg, *(const v4i*)(add_row + j * 512 + c * 8));
 #pragma unroll
       for (int d = 0; d < 4; ++d) {
         const unsigned w = (unsigned)seg[d];

@@ -223,6 +223,20 @@ class W4A4DecoderLayer(torch.nn.Module):
         self._tap(stage + ".scales", s.reshape(-1, s.size(-1)))
         return s, z, q
 
+    def _residual_norm_quant(self, stage, norm, norm_name, quantizer, x, add):
+        """(x + add, scales, zeros, codes): the residual addition (when `add` is given), the norm and the quantiser of
+        the linears that follow -- one launch where the whole-row path allows it, else the separate steps."""
+        if add is None:
+            return (x,) + tuple(self._norm_quant(stage, norm, norm_name, quantizer, x))
+        k = x.size(-1)
+        if self.activation == "token" and self.fused and self.record is None and k in (512, 1024, 2048, 4096, 8192):
+            total, q, s = _ops().add_rmsnorm_rotate_and_quantize_i4(
+                x.reshape(-1, k).contiguous(), add.reshape(-1, k).contiguous(), self._norm_weight16(norm_name, norm),
+                norm.eps)
+            return total.view(x.shape), s.view(*x.shape[:-1], 1), None, q.view(*x.shape[:-1], -1)
+        x = x + add
+        return (x,) + tuple(self._norm_quant(stage, norm, norm_name, quantizer, x))
+
     def _project(self, layers, q, s, z):
         if self.fused:
             return LinearFLH.forward_many(layers, q, s)
@@ -233,8 +247,14 @@ class W4A4DecoderLayer(torch.nn.Module):
         kv_cache: None, a pair (keys, values) [B, kv_heads, past, head_dim] that grows by concatenation, or one layer
         of a StaticKVCache together with `positions` (device int64 [T]: the slots the new tokens take; the cache's
         kv_len says how many slots attention reads).  Causal over past + T positions."""
+        _, y, cache = self._attention(x, None, cos, sin, kv_cache, positions)
+        return y, cache
+
+    def _attention(self, x, add, cos, sin, kv_cache=None, positions=None):
+        """attention() on the residual stream x + add (add may be None); returns that sum as well."""
         b, t, _ = x.shape
-        s, z, q = self._norm_quant("attn_in", self.input_layernorm, "input_layernorm", self.attn_quantizer1, x)
+        x, s, z, q = self._residual_norm_quant("attn_in", self.input_layernorm, "input_layernorm", self.attn_quantizer1,
+                                               x, add)
         qs, ks, vs = self._project([self.q_proj, self.k_proj, self.v_proj], q, s, z)
         self._tap("q_proj", qs), self._tap("k_proj", ks), self._tap("v_proj", vs)
         static = isinstance(kv_cache, StaticKVCache._Layer)
@@ -275,11 +295,11 @@ class W4A4DecoderLayer(torch.nn.Module):
         if (self.activation == "token" and self.fused and self.record is None and b * t <= 2
                 and self.hidden_size == 4096):
             # decode: the quantiser runs inside the GEMM's own launch (same bits as the two launches)
-            return self.o_proj.forward_online(out, hadamard="exact"), cache
+            return x, self.o_proj.forward_online(out, hadamard="exact"), cache
         s, z, q = self._token_quant("attn_out", out) if self.activation == "token" else self._group_quant("attn_out", self.attn_quantizer2, out)
         y = self.o_proj(q, s, z, x_is_packed=True)
         self._tap("o_proj", y)
-        return y, cache
+        return x, y, cache
 
     def _swiglu_gemm_applies(self):
         g = self.gate_proj
@@ -294,29 +314,48 @@ class W4A4DecoderLayer(torch.nn.Module):
         return s, z, q
 
     def mlp(self, x):
-        s, z, q = self._norm_quant("mlp_in", self.post_attention_layernorm, "post_attention_layernorm",
-                                   self.mlp_quantizer1, x)
-        if (self.activation == "token" and self.fused and self.record is None and q.numel() // q.size(-1) > 64
+        return self._mlp(x, None)[1]
+
+    def _mlp(self, x, add):
+        """mlp() on the residual stream x + add (add may be None); returns (that sum, the MLP's output)."""
+        x, s, z, q = self._residual_norm_quant("mlp_in", self.post_attention_layernorm, "post_attention_layernorm",
+                                               self.mlp_quantizer1, x, add)
+        rows = q.numel() // q.size(-1)
+        if (self.activation == "token" and self.fused and self.record is None and rows > 64
                 and self._swiglu_gemm_applies()):
             # prefill: gate and up in one launch that stores silu(gate) * up only (no fp16 [M, I] round trips)
             s, z, q = self._token_quant("mlp_mid", LinearFLH.forward_swiglu(self.gate_proj, self.up_proj, q, s))
-            return self.down_proj(q, s, z, x_is_packed=True)
+            return x, self.down_proj(q, s, z, x_is_packed=True)
         gate, up = self._project([self.gate_proj, self.up_proj], q, s, z)
         self._tap("gate_proj", gate), self._tap("up_proj", up)
-        if self.activation == "token":
-            s, z, q = self._token_quant("mlp_mid", torch.nn.functional.silu(gate) * up)
+        if (self.activation == "token" and self.fused and self.record is None and rows <= 256
+                and self.intermediate_size in (11008, 14336)):
+            # decode: silu(gate) * up formed inside the rotation's launch, never stored
+            q, s = _ops().silu_mul_rotate_and_quantize_i4(gate.reshape(rows, -1), up.reshape(rows, -1))
+            s, z, q = s.view(*x.shape[:-1], 1), None, q.view(*x.shape[:-1], -1)
+        elif self.activation == "token":
+            # (the library's product kernel when fused, so that every fused path sees the same fp16 product)
+            mid = _ops().silu_mul(gate, up) if self.fused else torch.nn.functional.silu(gate) * up
+            s, z, q = self._token_quant("mlp_mid", mid)
         elif self.fused and self.record is None:
             s, z, q = self._silu_mul_quant(gate, up)
         else:
             s, z, q = self._group_quant("mlp_mid", self.mlp_quantizer2, torch.nn.functional.silu(gate) * up)
         y = self.down_proj(q, s, z, x_is_packed=True)
         self._tap("down_proj", y)
-        return y
+        return x, y
 
     def forward(self, x, cos, sin, kv_cache=None, positions=None):
-        attn, cache = self.attention(x, cos, sin, kv_cache, positions)
-        x = x + attn
-        return x + self.mlp(x), cache
+        x, pending, cache = self.forward_deferred(x, None, cos, sin, kv_cache, positions)
+        return x + pending, cache
+
+    def forward_deferred(self, x, pending, cos, sin, kv_cache=None, positions=None):
+        """The layer on the residual stream x + pending, with its own last addition left to the caller: returns
+        (stream, pending, cache) with the layer's output = stream + pending.  A stack of layers passes the pair on, so that
+        every residual addition runs inside the launch of the norm + quantiser that reads its result."""
+        x, attn, cache = self._attention(x, pending, cos, sin, kv_cache, positions)
+        x, y = self._mlp(x, attn)
+        return x, y, cache
 
 
 def _ops():

@@ -96,8 +96,12 @@ class W4A4LlamaModel(torch.nn.Module):
         attention may read (>= positions.max() + 1).  Returns logits [B, T, vocab] fp16 (or the final hidden state)."""
         x = self.embed(input_ids)
         cos, sin = rotary_tables(positions, self.shape.head_dim, self.shape.rope_theta)
+        pending = None            # the last MLP output, added inside the next layer's first launch
         for i, layer in enumerate(self.layers):
-            x, _ = layer(x, cos, sin, cache.layer(i) if cache is not None else None, positions)
+            x, pending, _ = layer.forward_deferred(x, pending, cos, sin, cache.layer(i) if cache is not None else None,
+                                                   positions)
+        if pending is not None:
+            x = x + pending
         x = self.norm(x)
         return x if return_hidden else self.lm_head(x)
 

@@ -232,6 +232,28 @@ int flh_rotate_quant_i4(const flh_half* x, uint8_t* q_packed, flh_half* scales, 
                         uint32_t M, uint32_t K, int hadamard, int had_group, int scale_group,
                         float clip_ratio, void* stream);
 
+/* The residual addition in front of flh_rmsnorm_rotate_quant_i4: sum_out = fp16(x + add) row by row (one rounding per
+ * value, torch's fp16 addition), then exactly flh_rmsnorm_rotate_quant_i4(sum_out, ...) -- x, add, sum_out [M, K] fp16 (sum_out
+ * overlaps neither input), K = 512 .. 8192 a power of two, hadamard FLH_HAD_NONE or FLH_HAD_F32.  A decoder layer's
+ * "hidden = residual + attn; residual = hidden; hidden = norm(hidden)" followed by the quantiser of the next linears
+ * (flh/quantized_model/modeling_llama.py:600-618) in one launch instead of three.  Same bytes as the separate launches. */
+int flh_add_rmsnorm_rotate_quant_i4(const flh_half* x, const flh_half* add, flh_half* sum_out, const flh_half* weight,
+                                    float eps, uint8_t* q_packed, flh_half* scales, uint32_t M, uint32_t K, int hadamard,
+                                    float clip_ratio, void* stream);
+
+/* The SwiGLU product in front of the online rotation of down_proj, for decode-sized batches (M <= 256; prefill takes
+ * flh_gemm_i4_swiglu_o16): x = fp16(fp16(silu(gate)) * up) row by row, then exactly flh_rotate_quant_i4(x, ..., FLH_HAD_MFMA,
+ * one scale per row) -- gate, up [M, K] fp16 with K = 11008 (172 x 64) or 14336 (28 x 512); q_packed [M, K/2], scales [M].
+ * The product is formed in LDS and never stored.  The reference runs act_fn(gate) * up as torch kernels in front of its
+ * quantiser (flh/quantized_model/modeling_llama.py:522-526) and the online rotation of down_proj in front of that
+ * (fake_quant/main.py:30-35).  Same codes and scales as the separate launches on the same fp16 product. */
+int flh_silu_mul_rotate_quant_i4(const flh_half* gate, const flh_half* up, uint8_t* q_packed, flh_half* scales,
+                                 uint32_t M, uint32_t K, void* stream);
+
+/* The same product on its own: out[i] = fp16(fp16(silu(gate[i])) * up[i]) for n fp16 values (n a multiple of 8; out may
+ * be gate or up).  One launch for the two torch kernels of modeling_llama.py:522-526 where no quantiser follows directly. */
+int flh_silu_mul_f16(const flh_half* gate, const flh_half* up, flh_half* out, uint64_t n, void* stream);
+
 /* ---------------------------------------------------------------------------------
  * Between the q / k / v GEMM and attention of a decode (or prefill) step: rotary position embedding of the query and
  * key heads and the write of the new keys / values into a preallocated cache, one launch.  No native counterpart in the

@@ -212,6 +212,29 @@ def test_llama3_decode_step_against_the_oracle(llama3_two_layers, batch):
     assert err < 0.3
 
 
+@pytest.mark.parametrize("tokens", [1, 24, 600])
+def test_residual_additions_inside_the_next_launch_change_no_bit(llama3_two_layers, tokens):
+    """The stack hands (stream, pending addition) from layer to layer, so that every residual addition runs inside the
+    norm + quantiser launch that reads it; layer by layer with torch's additions in between must give the same bits
+    (decode-sized, short and prefill-sized row counts take different kernels)."""
+    model, _ = llama3_two_layers
+    shape = model.shape
+    gen = torch.Generator(device="cuda").manual_seed(tokens)
+    ids = torch.randint(0, shape.vocab_size, (1, tokens), device="cuda", generator=gen)
+    pos = torch.arange(tokens, device="cuda")
+    print(f"case deferred residual tokens={tokens}", flush=True)
+    with torch.no_grad():
+        got = model(ids, pos, None, return_hidden=True)
+        x = model.embed(ids)
+        cos, sin = rotary_tables(pos, shape.head_dim, shape.rope_theta)
+        for layer in model.layers:
+            attn, _ = layer.attention(x, cos, sin)
+            x = x + attn
+            x = x + layer.mlp(x)
+        want = model.norm(x)
+    assert torch.equal(got, want)
+
+
 def test_llama3_decode_step_replays_from_a_graph(llama3_two_layers):
     """The whole step (two layers, norm, head) captured once and replayed: the same logits as the eager step, on
     every replay, also after the token and the cache contents change between replays."""

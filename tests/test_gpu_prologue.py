@@ -223,3 +223,31 @@ def test_rmsnorm_rotate_short_batches_give_the_long_batch_bytes(ops):
         for rows in (1, 8, 16, 300, 512):
             q, s = ops.rmsnorm_rotate_and_quantize_i4(x[:rows].contiguous(), weight, 1e-5)
             assert torch.equal(q, q_long[:rows]) and torch.equal(s, s_long[:rows]), rows
+
+
+@pytest.mark.parametrize("k", [512, 4096, 8192])
+@pytest.mark.parametrize("m", [1, 5, 512, 700])
+@pytest.mark.parametrize("had", [True, False])
+def test_residual_add_in_front_of_rmsnorm_rotate_gives_the_separate_launches_bytes(ops, k, m, had):
+    """x + add in fp16 is one correctly rounded addition per value on the device as in torch, so the fused launch must
+    give torch's sum and, from it, the bytes of the launch without the addition (both row layouts: eight waves per row up
+    to 512 rows of 4096, one wave per row otherwise)."""
+    print(f"case add_rmsnorm m={m} k={k} had={had}", flush=True)
+    x = dev(syn.activations(m, k, seed=k + m))
+    add = dev((np.random.default_rng(m).standard_normal((m, k)) * 0.3).astype(np.float16))
+    w = dev(np.random.default_rng(3).uniform(0.5, 1.5, k).astype(np.float16))
+    total, q, s = ops.add_rmsnorm_rotate_and_quantize_i4(x, add, w, 1e-5, had)
+    assert torch.equal(total, x + add)
+    assert np.array_equal(host(total), (host(x).astype(np.float64) + host(add).astype(np.float64)).astype(np.float16))
+    q_ref, s_ref = ops.rmsnorm_rotate_and_quantize_i4(total, w, 1e-5, had)
+    assert torch.equal(q, q_ref) and torch.equal(s.view(torch.int16), s_ref.view(torch.int16))
+
+
+def test_residual_add_argument_errors(ops):
+    x = torch.zeros(4, 4096, dtype=torch.float16, device="cuda")
+    with pytest.raises(RuntimeError):
+        ops.add_rmsnorm_rotate_and_quantize_i4(x, x[:2], None, 1e-5)
+    with pytest.raises(RuntimeError):
+        ops.add_rmsnorm_rotate_and_quantize_i4(x[:, :768].contiguous(), x[:, :768].contiguous(), None, 1e-5)
+    with pytest.raises(RuntimeError):
+        ops.add_rmsnorm_rotate_and_quantize_i4(x, x.float(), None, 1e-5)
