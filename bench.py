@@ -37,7 +37,8 @@ PEAK_INT8_TOPS = 5033.0   # 256 CU x 8192 int8 op/clk/CU x 2.4 GHz (dense)
 PEAK_HBM_GBS = 8000.0
 # measured HBM traffic per launch at M = 2048 (fetch + write), from the counter runs summarised in
 # profiles/llama7b_block_M2048_hbm_traffic.txt
-GEMM_TRAFFIC_BYTES = int(((4 * 40.2 + 2 * 80.3 + 88.2) / 7 + (5 * 16.0 + 2 * 43.0) / 7) * 2 ** 20)
+GEMM_TRAFFIC_BYTES = {"seven": int(((4 * 40.2 + 2 * 80.3 + 88.2) / 7 + (5 * 16.0 + 2 * 43.0) / 7) * 2 ** 20),
+                      "layer": None}
 QUANT4096_TRAFFIC_BYTES = int((16.2 + 4.02) * 2 ** 20)
 
 # (name, N, K, activation source) -- activation sources are quantised once and shared
@@ -107,6 +108,9 @@ def main():
                     help="also launch three elementwise passes over 256 MiB (read 256 MiB, write 256 MiB): the "
                          "known-size kernel that hardware-counter readings (FETCH_SIZE / WRITE_SIZE) are scaled by")
     ap.add_argument("--hadamard", choices=["mixed", "exact", "fast"], default="fast")
+    ap.add_argument("--launches", choices=["layer", "seven"], default="layer",
+                    help="GEMM launches of the timed step: the four a decoder layer issues (q/k/v in one launch, gate and "
+                         "up in one launch that stores silu(gate)*up), or one per linear; the other form is reported beside it")
     ap.add_argument("--large-tokens", type=int, default=16384,
                     help="token count of the extra Hadamard-quant launches that amortise the launch floor")
     args = ap.parse_args()
@@ -131,37 +135,70 @@ def main():
             return "exact" if k & (k - 1) == 0 else "fast"
         return args.hadamard
 
-    def step(events=None):
-        packed = {}
-        for name in SOURCES:
-            if events is not None:
-                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-                e0.record()
-            packed[name] = ops.rotate_and_quantize_i4(acts[name], hadamard=had_mode(SOURCES[name]))
-            if events is not None:
-                e1.record()
-                events.append(("quant", name, e0, e1))
-        out = None
-        for name, n, k, src in LAYERS:
-            q, s = packed[src]
-            if events is not None:
-                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-                e0.record()
-            out = ops.gemm_i4_dequant_o16(q, weights[name][0], s, weights[name][1])
-            if events is not None:
-                e1.record()
-                events.append(("gemm", name, e0, e1))
-        return out
+    # The launches of one step.  "layer": what a decoder layer issues (flh_amd.quantized_model) -- q / k / v as three
+    # weight matrices of one launch, o, gate and up as one launch that stores silu(gate) * up, down: the same seven
+    # contractions in four GEMM launches.  "seven": one launch per linear.
+    FORMS = {"layer": [("qkv", "attn_in", ["q", "k", "v"]), ("o", "attn_out", ["o"]),
+                       ("gate_up_swiglu", "mlp_in", ["gate", "up"]), ("down", "mlp_mid", ["down"])],
+             "seven": [(name, src, [name]) for name, _, _, src in LAYERS]}
+    shape_of = {name: (n, k) for name, n, k, _ in LAYERS}
 
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    torch.cuda.synchronize()
-    dt = time.perf_counter() - t0
-    ms_per_step = dt / args.steps * 1e3
+    def launch(parts, q, s):
+        if len(parts) == 1:
+            return ops.gemm_i4_dequant_o16(q, weights[parts[0]][0], s, weights[parts[0]][1])
+        if parts == ["gate", "up"]:
+            return ops.gemm_i4_swiglu(q, weights["gate"][0], weights["up"][0], s, weights["gate"][1], weights["up"][1])
+        return ops.gemm_i4_dequant_multi(q, [weights[n][0] for n in parts], s, [weights[n][1] for n in parts])
+
+    def make_step(form):
+        def step(events=None):
+            packed = {}
+            for name in SOURCES:
+                if events is not None:
+                    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                    e0.record()
+                packed[name] = ops.rotate_and_quantize_i4(acts[name], hadamard=had_mode(SOURCES[name]))
+                if events is not None:
+                    e1.record()
+                    events.append(("quant", name, e0, e1))
+            out = None
+            for name, src, parts in FORMS[form]:
+                q, s = packed[src]
+                if events is not None:
+                    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                    e0.record()
+                out = launch(parts, q, s)
+                if events is not None:
+                    e1.record()
+                    events.append(("gemm", name, e0, e1))
+            return out
+        return step
+
+    def run_form(form):
+        """(ms per step over exactly --steps steps after --warmup, median us per launch from a second pass with HIP
+        events on the launch stream around every launch)"""
+        step = make_step(form)
+        for _ in range(args.warmup):
+            step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            step()
+        torch.cuda.synchronize()
+        ms = (time.perf_counter() - t0) / args.steps * 1e3
+        events = []
+        for _ in range(args.steps):
+            step(events)
+        torch.cuda.synchronize()
+        per = {}
+        for kind, name, e0, e1 in events:
+            per.setdefault((kind, name), []).append(e0.elapsed_time(e1) * 1e3)  # us
+        return ms, {k: float(np.median(v)) for k, v in per.items()}
+
+    other_form = "seven" if args.launches == "layer" else "layer"
+    ms_other, med_other = run_form(other_form)
+    ms_per_step, med = run_form(args.launches)      # the headline: timed last, on a warm device
+    step = make_step("seven")
 
     # The same step with the weights of projections that share an input stored concatenated ([q; k; v] and
     # [gate; up], as a model loader may lay them out): identical outputs from four GEMM launches instead of
@@ -187,16 +224,6 @@ def main():
     ms_concat = (time.perf_counter() - t0) / args.steps * 1e3
     del cat_w
 
-
-    # per-kernel durations: HIP events on the launch stream around every launch of a second timed pass
-    events = []
-    for _ in range(args.steps):
-        step(events)
-    torch.cuda.synchronize()
-    per = {}
-    for kind, name, e0, e1 in events:
-        per.setdefault((kind, name), []).append(e0.elapsed_time(e1) * 1e3)  # us
-    med = {k: float(np.median(v)) for k, v in per.items()}
 
     # ... and with the weights left where they are: the projections that share an input go through the entry point
     # that takes several weight matrices (gemm_i4_dequant_multi), again four GEMM launches, identical outputs
@@ -743,8 +770,17 @@ def main():
         del src, dst
 
     total_ops = sum(gemm_ops(M, n, k) for _, n, k, _ in LAYERS)
-    gemm_us = sum(med[("gemm", name)] for name, *_ in LAYERS)
+    launches = FORMS[args.launches]
+    gemm_us = sum(med[("gemm", name)] for name, *_ in launches)
     gemm_tops = total_ops / (gemm_us * 1e-6) / 1e12
+
+    def launch_table(form, m):
+        out = {}
+        for name, _, parts in FORMS[form]:
+            o = sum(gemm_ops(M, *shape_of[n]) for n in parts)
+            out[name] = {"us": round(m[("gemm", name)], 2), "TOPS": round(o / (m[("gemm", name)] * 1e-6) / 1e12, 1)}
+        return out
+    other_us = sum(med_other[("gemm", name)] for name, *_ in FORMS[other_form])
     quant_detail = {}
     for name, k in SOURCES.items():
         us = med[("quant", name)]
@@ -762,16 +798,25 @@ def main():
         "dtype": "int4 codes on int8 MFMA, int32 accumulate, fp32/fp16 epilogue",
         "data": "synthetic",
         "config": {"workload": "Llama-2-7B decoder-block linears, M=2048, per-token x per-channel scales "
-                               "(the configuration the headline metric is quoted on)", "tokens": M},
-        "roofline": {"bound": "mfma", "kernel": "gemm_i4_kernel (row-scale epilogue), 7 launches per step",
+                               "(the configuration the headline metric is quoted on)", "tokens": M,
+                   "launches": args.launches},
+        "roofline": {"bound": "mfma",
+                     "kernel": "gemm_i4_kernel (row-scale epilogue), " +
+                               ("4 launches per step: q/k/v in one, o, gate and up in one (stores silu(gate)*up), down"
+                                if args.launches == "layer" else "7 launches per step"),
                      "achieved": round(gemm_tops, 1), "peak": PEAK_INT8_TOPS, "unit": "TOP/s",
                      "frac": round(gemm_tops / PEAK_INT8_TOPS, 4),
                      # HBM bytes per launch averaged over the seven launches (rocprofv3 --pmc FETCH_SIZE and
                      # WRITE_SIZE runs of this script, calibrated on a 256 MiB copy; summary under profiles/)
-                     "traffic": GEMM_TRAFFIC_BYTES if M == 2048 else None,
-                     "avg_launch_us": round(gemm_us / len(LAYERS), 2),
-                     "per_launch_us": {name: round(med[("gemm", name)], 2) for name, *_ in LAYERS},
+                     "traffic": GEMM_TRAFFIC_BYTES[args.launches] if M == 2048 else None,
+                     "avg_launch_us": round(gemm_us / len(launches), 2),
+                     "per_launch": launch_table(args.launches, med),
                      },
+        f"launches={other_form}": {"us_per_layer": round(ms_other * 1e3, 1),
+                                   "TOPS": round(total_ops / (ms_other * 1e-3) / 1e12, 2),
+                                   "gemm_TOP/s": round(total_ops / (other_us * 1e-6) / 1e12, 1),
+                                   "gemm_frac_of_peak": round(total_ops / (other_us * 1e-6) / 1e12 / PEAK_INT8_TOPS, 4),
+                                   "per_launch": launch_table(other_form, med_other)},
         "roofline_hadamard_quant": {"bound": "hbm",
                                     "kernel": ("rotate_quant_mfma4096_kernel" if had_mode(4096) == "fast" else
                                                "rotate_quant_wave_kernel<8>") + f" (K=4096, M={M}, inside the step)",
