@@ -58,6 +58,7 @@ _SIG = {
     "flh_decode_attention_workspace_bytes": (_c.c_size_t, [_c.c_uint32, _c.c_uint32, _c.c_uint32, _c.c_uint32]),
     "flh_decode_attention_f16": (_c.c_int, [_PTR, _PTR, _PTR, _PTR, _c.c_uint32, _c.c_uint32, _c.c_uint32, _c.c_uint32,
                                             _c.c_uint32, _c.c_uint32, _c.c_float, _PTR, _c.c_size_t, _PTR]),
+    "flh_decode_attention_rope_f16": (_c.c_int, [_PTR] * 9 + [_c.c_uint32] * 6 + [_c.c_float, _PTR, _c.c_size_t, _PTR]),
     "flh_decode_attention_static_scratch_bytes": (_c.c_size_t, []),
     "flh_decode_attention_f16_static": (_c.c_int, [_PTR, _PTR, _PTR, _PTR, _c.c_uint32, _c.c_uint32, _c.c_uint32,
                                                    _c.c_uint32, _c.c_uint32, _c.c_uint32, _c.c_float, _PTR]),

@@ -400,6 +400,47 @@ def decode_attention(q, k_cache, v_cache, kv_len, scale=None, workspace=None):
     return out
 
 
+def decode_attention_rope(q, k_new, v_new, cos, sin, positions, k_cache, v_cache, kv_len, scale=None, workspace=None):
+    """decode_attention with the rotary embedding and the cache write of the new token inside: q [B, Hq, d], k_new /
+    v_new [B, Hkv, d] fp16 as projected (not rotated), cos / sin [1, d] or [d] fp16 of the new position, positions (int64
+    CUDA tensor, first element = the cache slot of the new token, < kv_len) -> [B, Hq, d] fp16.  k_cache / v_cache receive
+    the rotated key and the value at that slot (the bytes rope_kv_cache_ would write); q is not modified."""
+    for t_ in (q, k_new, v_new, cos, sin, k_cache, v_cache):
+        _check(t_.is_cuda and t_.dtype == torch.float16 and t_.is_contiguous() and t_.device == q.device,
+               "tensors must be contiguous float16 CUDA tensors on one device")
+    _check(q.dim() == 3 and k_cache.dim() == 4 and k_cache.shape == v_cache.shape and k_cache.size(0) == q.size(0)
+           and k_cache.size(3) == q.size(2), "q [B, Hq, d] and caches [B, Hkv, max_len, d] expected")
+    B, Hq, d = q.shape
+    Hkv, max_len = k_cache.size(1), k_cache.size(2)
+    _check(k_new.shape == (B, Hkv, d) and v_new.shape == (B, Hkv, d), "k_new / v_new [B, Hkv, d] expected")
+    _check(cos.numel() == d and sin.numel() == d, "cos / sin of one position (d values each) expected")
+    _check(positions.is_cuda and positions.dtype == torch.int64 and positions.numel() >= 1 and positions.device == q.device,
+           "positions must be an int64 CUDA tensor")
+    _check(d in (64, 128), "head_dim must be 64 or 128")
+    _check(Hkv > 0 and Hq % Hkv == 0 and Hq // Hkv in (1, 2, 4, 8), "Hq / Hkv must be 1, 2, 4 or 8")
+    _check(0 < kv_len <= max_len, "kv_len must be in 1 .. max_len")
+    out = torch.empty_like(q)
+    if B == 0:
+        return out
+    need = int(_lib.load().flh_decode_attention_workspace_bytes(B, Hq, d, int(kv_len)))
+    if workspace is None:
+        key = (q.device.index, _stream(q))
+        workspace = _attention_workspaces.get(key)
+        if workspace is None or workspace.numel() < need:
+            _check(not torch.cuda.is_current_stream_capturing(),
+                   "decode_attention: call it once eagerly (or pass a workspace) before capturing a graph")
+            workspace = torch.empty(max(need, 1 << 20), dtype=torch.uint8, device=q.device)
+            _attention_workspaces[key] = workspace
+    else:
+        _check(workspace.is_cuda and workspace.dtype == torch.uint8 and workspace.is_contiguous()
+               and workspace.device == q.device and workspace.numel() >= need, f"workspace: {need} bytes of uint8 needed")
+    _run("flh_decode_attention_rope_f16", q.device, q.data_ptr(), k_new.data_ptr(), v_new.data_ptr(), cos.data_ptr(),
+         sin.data_ptr(), positions.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(), B, Hq, Hkv, d,
+         int(kv_len), max_len, float(scale if scale is not None else d ** -0.5), workspace.data_ptr(), workspace.numel(),
+         _stream(q))
+    return out
+
+
 def _check_rows(x, width):
     _check(x.is_cuda, "Input tensor must be on CUDA")
     _check(x.dtype == torch.float16, "Input tensor must be float16 (half)")

@@ -21,52 +21,115 @@ constexpr int kAttnThreads = 256;
 template <int D>
 constexpr int partial_floats(int rep) { return rep * (D + 2); }
 
-template <int D, int REP, int CHUNK>
+// One value of the rotary embedding with the roundings of the tensor expression x * cos + rotate_half(x) * sin evaluated
+// op by op in fp16 (the same as the stand-alone kernel, rope_cache.hip): `first_half` says whether x sits in the first
+// half of the head vector (its partner xp then enters negated).
+__device__ __forceinline__ _Float16 rope_value(_Float16 x, _Float16 xp, _Float16 c, _Float16 s, bool first_half) {
+  const _Float16 a = (_Float16)round_here((float)x * (float)c);
+  const _Float16 r = (_Float16)round_here((first_half ? -1.f : 1.f) * (float)xp * (float)s);
+  return (_Float16)round_here((float)a + (float)r);
+}
+
+// ROPE: the step's new token comes in un-rotated -- q, and k_new / v_new [B, Hkv, D] -- together with the cos / sin row of
+// its position and the cache slot `positions[0]` it takes (the same for every sequence).  The queries are rotated while
+// they are loaded; the workgroup whose chunk holds the slot rotates the new key, uses it and the new value in place of
+// what the cache holds there, and writes both into the cache.  One launch less in front of attention, and the same
+// bytes in the cache as the stand-alone rotary / cache kernel writes.
+template <int D, int REP, int CHUNK, bool ROPE>
 __global__ __launch_bounds__(kAttnThreads) void decode_attention_partial_kernel(
-    const __half* __restrict__ q, const __half* __restrict__ k_cache, const __half* __restrict__ v_cache,
-    float* __restrict__ partials, uint32_t Hkv, uint32_t kv_len, uint32_t max_len, uint32_t splits, float scale) {
+    const __half* __restrict__ q, __half* k_cache, __half* v_cache, float* __restrict__ partials, uint32_t Hkv,
+    uint32_t kv_len, uint32_t max_len, uint32_t splits, float scale, const __half* __restrict__ k_new,
+    const __half* __restrict__ v_new, const __half* __restrict__ cos, const __half* __restrict__ sin,
+    const long long* __restrict__ positions) {
   static_assert(D == 128 || D == 64, "head dimension");
   static_assert(CHUNK == 64, "one key per lane in the softmax step");
   constexpr int TPK = kAttnThreads / CHUNK;            // threads per key: 4
   constexpr int CPT = D / TPK;                         // channels per thread in the score step: 32 (16)
+  constexpr int RPW = CHUNK / (kAttnThreads / 64);     // value rows per wave: 16
   __shared__ float qs[REP * D];                        // the query heads as float
   __shared__ float sc[REP][CHUNK];                     // scores, then probabilities
+  __shared__ float red[kAttnThreads / 64][REP * D];    // the waves' weighted values
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const uint32_t split = blockIdx.x % splits, bh = blockIdx.x / splits;   // bh = b * Hkv + kvh
   const uint32_t t0 = split * CHUNK;
+  uint32_t slot = 0xFFFFFFFFu;                         // cache slot of the new token (ROPE), if it is inside kv_len
+  if constexpr (ROPE) {
+    const long long pos = positions[0];
+    if (pos >= 0 && pos < (long long)kv_len) slot = (uint32_t)pos;
+  }
   const __half* qh = q + (size_t)bh * REP * D;         // q [B, Hq, D]: the REP heads of this kv head are adjacent
-  for (int i = tid; i < REP * D; i += kAttnThreads) qs[i] = __half2float(qh[i]);
-  __syncthreads();
+  for (int i = tid; i < REP * D; i += kAttnThreads) {
+    if constexpr (ROPE) {
+      const int d = i % D;
+      const _Float16 *qf = (const _Float16*)qh, *cf = (const _Float16*)cos, *sf = (const _Float16*)sin;
+      qs[i] = (float)rope_value(qf[i], qf[i ^ (D / 2)], cf[d], sf[d], d < D / 2);
+    } else {
+      qs[i] = __half2float(qh[i]);
+    }
+  }
 
   // scores: thread (key, part) takes CPT channels of its key
   const int key = tid / TPK, part = tid % TPK;
   const uint32_t t = t0 + key;
   const bool live = t < kv_len;
-  const __half* kr = k_cache + ((size_t)bh * max_len + (live ? t : 0)) * D + part * CPT;
   float kv[CPT];
+  if (ROPE && t == slot) {                             // the new key: rotate it, keep it, and store it in its slot
+    const __half* src = k_new + (size_t)bh * D;
+    const int c0 = part * CPT, p0 = c0 ^ (D / 2);
+    __half* dst = k_cache + ((size_t)bh * max_len + t) * D + c0;
 #pragma unroll
-  for (int c8 = 0; c8 < CPT / 8; ++c8) {
-    const h8 v = *(const h8*)(kr + c8 * 8);
+    for (int c8 = 0; c8 < CPT / 8; ++c8) {
+      const h8 x = *(const h8*)(src + c0 + c8 * 8), xp = *(const h8*)(src + p0 + c8 * 8);
+      const h8 cc = *(const h8*)(cos + c0 + c8 * 8), ss = *(const h8*)(sin + c0 + c8 * 8);
+      h8 y;
 #pragma unroll
-    for (int e = 0; e < 8; ++e) kv[c8 * 8 + e] = (float)v[e];
+      for (int e = 0; e < 8; ++e) {
+        y[e] = rope_value(x[e], xp[e], cc[e], ss[e], c0 < D / 2);
+        kv[c8 * 8 + e] = (float)y[e];
+      }
+      *(h8*)(dst + c8 * 8) = y;
+    }
+  } else {
+    const __half* kr = k_cache + ((size_t)bh * max_len + (live ? t : 0)) * D + part * CPT;
+#pragma unroll
+    for (int c8 = 0; c8 < CPT / 8; ++c8) {
+      const h8 v = *(const h8*)(kr + c8 * 8);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) kv[c8 * 8 + e] = (float)v[e];
+    }
   }
-  // this lane's channel pair (channel for D = 64) of every value row of the chunk, requested now: the loads travel
-  // while the scores and the softmax pieces are computed
+  // Values: wave w takes rows 16 w .. 16 w + 15 of the chunk, a lane one channel pair (one channel for D = 64) of
+  // each; requested now, the loads travel while the scores and the softmax pieces are computed.
   const uint32_t n_live = kv_len > t0 ? min((uint32_t)CHUNK, kv_len - t0) : 0u;
-  const __half* vr = v_cache + ((size_t)bh * max_len + t0) * D;
-  float vv0[CHUNK], vv1[D == 128 ? CHUNK : 1];
+  __half* vr = v_cache + ((size_t)bh * max_len + t0 + wave * RPW) * D;
+  float vv0[RPW], vv1[D == 128 ? RPW : 1];
 #pragma unroll
-  for (int i = 0; i < CHUNK; ++i) {
+  for (int i = 0; i < RPW; ++i) {
+    const uint32_t row = wave * RPW + i;               // wave-uniform
+    const bool fresh = ROPE && t0 + row == slot;
     if constexpr (D == 128) {
       h2 v = {(_Float16)0.f, (_Float16)0.f};
-      if ((uint32_t)i < n_live) v = *(const h2*)(vr + (size_t)i * D + 2 * lane);
+      if (fresh) {
+        v = *(const h2*)(v_new + (size_t)bh * D + 2 * lane);
+        *(h2*)(vr + (size_t)i * D + 2 * lane) = v;
+      } else if (row < n_live) {
+        v = *(const h2*)(vr + (size_t)i * D + 2 * lane);
+      }
       vv0[i] = (float)v[0];
       vv1[i] = (float)v[1];
     } else {
-      vv0[i] = (uint32_t)i < n_live ? __half2float(vr[(size_t)i * D + lane]) : 0.f;
+      __half v = __float2half(0.f);
+      if (fresh) {
+        v = v_new[(size_t)bh * D + lane];
+        vr[(size_t)i * D + lane] = v;
+      } else if (row < n_live) {
+        v = vr[(size_t)i * D + lane];
+      }
+      vv0[i] = __half2float(v);
     }
   }
+  __syncthreads();                                     // the queries are in LDS
 #pragma unroll
   for (int h = 0; h < REP; ++h) {
     float s = 0.f;
@@ -78,8 +141,7 @@ __global__ __launch_bounds__(kAttnThreads) void decode_attention_partial_kernel(
   }
   __syncthreads();
 
-  // softmax pieces of this chunk, head h by wave h (REP > 4: two heads per wave), then the weighted values:
-  // lane = a channel pair, all waves walk over the same value rows
+  // softmax pieces of this chunk, head h by wave h (REP > 4: two heads per wave)
   float* out = partials + (size_t)blockIdx.x * partial_floats<D>(REP);
   for (int h = wave; h < REP; h += kAttnThreads / 64) {
     const float s = sc[h][lane];
@@ -93,17 +155,22 @@ __global__ __launch_bounds__(kAttnThreads) void decode_attention_partial_kernel(
     }
   }
   __syncthreads();
-  for (int h = wave; h < REP; h += kAttnThreads / 64) {
+  // weighted values: every wave its own rows for all heads, then the four waves' sums in a fixed order
+#pragma unroll
+  for (int h = 0; h < REP; ++h) {
     float a0 = 0.f, a1 = 0.f;
 #pragma unroll
-    for (int i = 0; i < CHUNK; ++i) {                  // probabilities past kv_len are zero, their values were not loaded
-      const float p = sc[h][i];
+    for (int i = 0; i < RPW; ++i) {                    // probabilities past kv_len are zero, their values were not loaded
+      const float p = sc[h][wave * RPW + i];
       a0 = __builtin_fmaf(p, vv0[i], a0);
       if constexpr (D == 128) a1 = __builtin_fmaf(p, vv1[i], a1);
     }
-    if constexpr (D == 128) *(v2f*)(out + h * (D + 2) + 2 * lane) = v2f{a0, a1};
-    else out[h * (D + 2) + lane] = a0;
+    if constexpr (D == 128) *(v2f*)(&red[wave][h * D + 2 * lane]) = v2f{a0, a1};
+    else red[wave][h * D + lane] = a0;
   }
+  __syncthreads();
+  for (int i = tid; i < REP * D; i += kAttnThreads)
+    out[(i / D) * (D + 2) + i % D] = (red[0][i] + red[1][i]) + (red[2][i] + red[3][i]);
 }
 
 // one workgroup of four waves per (sequence, query head): the chunks' partials -> fp16 output.  Every wave reads all
@@ -163,12 +230,23 @@ __global__ __launch_bounds__(256) void decode_attention_combine_kernel(const flo
 
 constexpr int kChunk = 64;
 
+// the new token's inputs of the variant with the rotary embedding and the cache write inside (all null without it)
+struct NewToken {
+  const __half *k, *v, *cos, *sin;
+  const long long* positions;
+};
+
 template <int D, int REP>
-int launch_attention(const __half* q, const __half* k, const __half* v, __half* out, float* partials, uint32_t B,
-                     uint32_t Hkv, uint32_t kv_len, uint32_t max_len, float scale, hipStream_t stream) {
+int launch_attention(const __half* q, __half* k, __half* v, __half* out, float* partials, uint32_t B, uint32_t Hkv,
+                     uint32_t kv_len, uint32_t max_len, float scale, const NewToken& nt, hipStream_t stream) {
   const uint32_t splits = (kv_len + kChunk - 1) / kChunk;
-  hipLaunchKernelGGL((decode_attention_partial_kernel<D, REP, kChunk>), dim3(B * Hkv * splits), dim3(kAttnThreads), 0, stream,
-                     q, k, v, partials, Hkv, kv_len, max_len, splits, scale);
+  const dim3 grid(B * Hkv * splits), block(kAttnThreads);
+  if (nt.k)
+    hipLaunchKernelGGL((decode_attention_partial_kernel<D, REP, kChunk, true>), grid, block, 0, stream, q, k, v, partials,
+                       Hkv, kv_len, max_len, splits, scale, nt.k, nt.v, nt.cos, nt.sin, nt.positions);
+  else
+    hipLaunchKernelGGL((decode_attention_partial_kernel<D, REP, kChunk, false>), grid, block, 0, stream, q, k, v, partials,
+                       Hkv, kv_len, max_len, splits, scale, nt.k, nt.v, nt.cos, nt.sin, nt.positions);
   if (int rc = check_launch("decode_attention (partials)")) return rc;
   hipLaunchKernelGGL((decode_attention_combine_kernel<D>), dim3(B * Hkv * REP), dim3(256), 0, stream, partials, out,
                      (uint32_t)REP, splits);
@@ -185,10 +263,10 @@ extern "C" size_t flh_decode_attention_workspace_bytes(uint32_t B, uint32_t Hq, 
   return (size_t)B * Hq * splits * (head_dim + 2) * sizeof(float);
 }
 
-extern "C" int flh_decode_attention_f16(const flh_half* q, const flh_half* k_cache, const flh_half* v_cache, flh_half* out,
-                                        uint32_t B, uint32_t Hq, uint32_t Hkv, uint32_t head_dim, uint32_t kv_len,
-                                        uint32_t max_len, float scale, void* workspace, size_t workspace_bytes,
-                                        void* stream) {
+namespace {
+int decode_attention_checked(const flh_half* q, flh_half* k_cache, flh_half* v_cache, flh_half* out, uint32_t B, uint32_t Hq,
+                             uint32_t Hkv, uint32_t head_dim, uint32_t kv_len, uint32_t max_len, float scale,
+                             void* workspace, size_t workspace_bytes, const NewToken& nt, void* stream) {
   if (!q || !k_cache || !v_cache || !out) return fail(FLH_EINVAL, "decode_attention: null pointer");
   if (misaligned16(q, k_cache, v_cache, out)) return fail(FLH_EINVAL, "decode_attention: tensors must be 16-byte aligned");
   if (head_dim != 128 && head_dim != 64) return fail(FLH_EINVAL, "decode_attention: head_dim (%u) must be 64 or 128", head_dim);
@@ -203,11 +281,11 @@ extern "C" int flh_decode_attention_f16(const flh_half* q, const flh_half* k_cac
   if (workspace_bytes < need)
     return fail(FLH_EINVAL, "decode_attention: the workspace has %zu bytes, this call needs %zu", workspace_bytes, need);
   if ((uint64_t)B * Hkv * ((kv_len + kChunk - 1) / kChunk) > 0x7FFFFFFFull) return fail(FLH_EINVAL, "decode_attention: too many chunks");
-  const __half *qh = (const __half*)q, *kh = (const __half*)k_cache, *vh = (const __half*)v_cache;
-  __half* oh = (__half*)out;
+  const __half* qh = (const __half*)q;
+  __half *kh = (__half*)k_cache, *vh = (__half*)v_cache, *oh = (__half*)out;
   float* ws = (float*)workspace;
   hipStream_t st = (hipStream_t)stream;
-#define FLH_ATTN(D, R) return launch_attention<D, R>(qh, kh, vh, oh, ws, B, Hkv, kv_len, max_len, scale, st)
+#define FLH_ATTN(D, R) return launch_attention<D, R>(qh, kh, vh, oh, ws, B, Hkv, kv_len, max_len, scale, nt, st)
   if (head_dim == 128) {
     switch (rep) {
       case 1: FLH_ATTN(128, 1);
@@ -223,6 +301,29 @@ extern "C" int flh_decode_attention_f16(const flh_half* q, const flh_half* k_cac
     default: FLH_ATTN(64, 8);
   }
 #undef FLH_ATTN
+}
+}  // namespace
+
+extern "C" int flh_decode_attention_f16(const flh_half* q, const flh_half* k_cache, const flh_half* v_cache, flh_half* out,
+                                        uint32_t B, uint32_t Hq, uint32_t Hkv, uint32_t head_dim, uint32_t kv_len,
+                                        uint32_t max_len, float scale, void* workspace, size_t workspace_bytes,
+                                        void* stream) {
+  // (without a new token the kernel only reads the caches)
+  return decode_attention_checked(q, (flh_half*)k_cache, (flh_half*)v_cache, out, B, Hq, Hkv, head_dim, kv_len, max_len, scale,
+                                  workspace, workspace_bytes, NewToken{nullptr, nullptr, nullptr, nullptr, nullptr}, stream);
+}
+
+extern "C" int flh_decode_attention_rope_f16(const flh_half* q, const flh_half* k_new, const flh_half* v_new,
+                                             const flh_half* cos, const flh_half* sin, const int64_t* positions,
+                                             flh_half* k_cache, flh_half* v_cache, flh_half* out, uint32_t B, uint32_t Hq,
+                                             uint32_t Hkv, uint32_t head_dim, uint32_t kv_len, uint32_t max_len, float scale,
+                                             void* workspace, size_t workspace_bytes, void* stream) {
+  if (!k_new || !v_new || !cos || !sin || !positions) return fail(FLH_EINVAL, "decode_attention (rotary): null pointer");
+  if (misaligned16(k_new, v_new, cos, sin)) return fail(FLH_EINVAL, "decode_attention (rotary): tensors must be 16-byte aligned");
+  return decode_attention_checked(q, k_cache, v_cache, out, B, Hq, Hkv, head_dim, kv_len, max_len, scale, workspace,
+                                  workspace_bytes,
+                                  NewToken{(const __half*)k_new, (const __half*)v_new, (const __half*)cos, (const __half*)sin,
+                                           (const long long*)positions}, stream);
 }
 
 // ---- the same for callers that cannot allocate ---------------------------------------------------------------------

@@ -36,7 +36,10 @@ class LinearFLH(torch.nn.Module):
         # second time, re-encoded at 6 bits per code; outputs are bit-identical.  Pays for wide layers and group scales.
         # The encoding is rebuilt whenever `w_packed` has been written to or replaced (in-place copies, load_state_dict,
         # .to(device)): it is keyed on the buffer's storage address and version counter.
-        self.six_bit = False
+        # The 6-bit matrix instruction for prefill-sized calls (same bits, no unpack in the loop; needs a second, 6-bit
+        # copy of the weights, built on first use): True / False, or None = where it is faster even with the pass that
+        # re-encodes the activations -- weights with a scale per group of 128.
+        self.six_bit = None
         self.six_bit_min_rows = 256
         self._w6 = None
         self._w6_key = None
@@ -52,11 +55,12 @@ class LinearFLH(torch.nn.Module):
         return self._w6
 
     def _six_bit_applies(self, rows, a_scale, w_scale, group):
-        if not (self.six_bit and rows.is_cuda and rows.size(0) >= self.six_bit_min_rows and self.in_features % 128 == 0):
+        if self.six_bit is False or not (rows.is_cuda and rows.size(0) >= self.six_bit_min_rows
+                                         and self.in_features % 128 == 0):
             return False
         per_row = a_scale.size(1) == 1 and w_scale.size(1) == 1
         grouped = group == 128 and w_scale.size(1) == self.in_features // 128 and a_scale.size(1) in (1, w_scale.size(1))
-        return per_row or grouped
+        return grouped or (per_row and self.six_bit is True)
 
     # ------------------------------------------------------------------ kernels
     def forward(self, x, a_scale=None, a_zero=None, x_is_packed=False, is_symmetric=None):

@@ -146,7 +146,7 @@ class W4A4DecoderLayer(torch.nn.Module):
 
     @classmethod
     def from_float(cls, weights, num_heads, num_kv_heads, eps=1e-5, act_group_size=128, weight_group_size=None,
-                   fused=True, activation="group", six_bit=False):
+                   fused=True, activation="group", six_bit=None):
         """weights: fp16 tensors `q_proj` ... `down_proj` [N, K] (as nn.Linear stores them) and optionally
         `input_layernorm` / `post_attention_layernorm` [hidden]; quantised round-to-nearest ("group": as they are,
         "token": after the rotation of their input side).  weight_group_size: None = 128 for "group" and one scale
@@ -171,9 +171,9 @@ class W4A4DecoderLayer(torch.nn.Module):
             src.weight.data.copy_(w)
             setattr(layer, name, LinearFLH.from_float(src, weight_group_size=weight_group_size,
                                                       in_group_size=act_group_size, no_hadamard=True))
-        if six_bit:        # prefill-sized calls run on the 6-bit matrix instruction (second encoding of the weights)
-            for name in cls.PROJECTIONS:
-                getattr(layer, name).six_bit = True
+        if six_bit is not None:   # True: prefill-sized calls on the 6-bit matrix instruction (second encoding of the
+            for name in cls.PROJECTIONS:   # weights); False: never; None: LinearFLH's own choice (group-scaled weights)
+                getattr(layer, name).six_bit = six_bit
         for name in ("input_layernorm", "post_attention_layernorm"):
             norm = getattr(layer, name).to(device)
             if name in weights:
@@ -259,18 +259,24 @@ class W4A4DecoderLayer(torch.nn.Module):
         self._tap("q_proj", qs), self._tap("k_proj", ks), self._tap("v_proj", vs)
         static = isinstance(kv_cache, StaticKVCache._Layer)
         out = None
-        if static:
+        if (static and t == 1 and self.head_dim in (64, 128) and self.num_heads // self.num_kv_heads in (1, 2, 4, 8)
+                and positions is not None):
+            # one new token against the cache: rotary embedding, cache write and chunked attention in two launches
+            keys, values = kv_cache.tensors()
+            out = _ops().decode_attention_rope(qs.view(b, self.num_heads, self.head_dim),
+                                               ks.view(b, self.num_kv_heads, self.head_dim),
+                                               vs.view(b, self.num_kv_heads, self.head_dim), cos, sin, positions, keys,
+                                               values, kv_cache.owner.kv_len,
+                                               workspace=kv_cache.owner.attention_workspace)
+            out = out.view(b, 1, self.hidden_size)
+            cache = kv_cache
+            past = kv_cache.owner.kv_len - 1
+        elif static:
             # rotary embedding of q (in place) and k, and the new keys / values into their cache slots: one launch
             qs = qs.view(b, t, self.num_heads, self.head_dim)
             ks, vs = kv_cache.rope_and_update(qs, ks.view(b, t, self.num_kv_heads, self.head_dim),
                                               vs.view(b, t, self.num_kv_heads, self.head_dim), cos, sin, positions)
             cache = kv_cache
-            if t == 1 and self.head_dim in (64, 128) and self.num_heads // self.num_kv_heads in (1, 2, 4, 8):
-                # one new token against the cache: the chunked decode-attention kernel (two launches)
-                keys, values = kv_cache.tensors()
-                out = _ops().decode_attention(qs.view(b, self.num_heads, self.head_dim), keys, values, ks.size(2),
-                                              workspace=kv_cache.owner.attention_workspace)
-                out = out.view(b, 1, self.hidden_size)
             qs = qs.transpose(1, 2)
         else:
             qs = qs.view(b, t, self.num_heads, self.head_dim).transpose(1, 2)
@@ -282,8 +288,8 @@ class W4A4DecoderLayer(torch.nn.Module):
                 ks, vs = torch.cat((kv_cache[0], ks), dim=2), torch.cat((kv_cache[1], vs), dim=2)
             cache = (ks, vs)
         gqa = self.num_heads != self.num_kv_heads
-        past = ks.size(2) - t
         if out is None:
+            past = ks.size(2) - t
             if t == 1 and past > 0:
                 out = _decode_attention(qs, ks, vs)           # one new token sees every cached position
             elif past == 0:
@@ -306,6 +312,15 @@ class W4A4DecoderLayer(torch.nn.Module):
         cols = g.w_scale.view(g.out_features, -1).size(1)
         return g.bias is None and self.up_proj.bias is None and (cols == 1 or (g.weight_group_size == 128 and cols == g.in_features // 128))
 
+    def _six_bit_gate_up(self, q, s):
+        """Whether gate / up would take the 6-bit matrix instruction for these activations (faster than the int8 launch
+        that fuses the SwiGLU product when the weights carry group scales)."""
+        rows = q.reshape(-1, q.size(-1))
+        g = self.gate_proj
+        group = g.weight_group_size if g.weight_group_size > 0 else (g.in_group_size or 128)
+        return all(l._six_bit_applies(rows, s.reshape(rows.size(0), -1), l.w_scale.view(l.out_features, -1), group)
+                   for l in (self.gate_proj, self.up_proj))
+
     def _group_quant(self, stage, quantizer, x):
         s, z, q = quantizer(x)
         self._tap(stage + ".input", x.reshape(-1, x.size(-1)))
@@ -322,7 +337,7 @@ class W4A4DecoderLayer(torch.nn.Module):
                                                self.mlp_quantizer1, x, add)
         rows = q.numel() // q.size(-1)
         if (self.activation == "token" and self.fused and self.record is None and rows > 64
-                and self._swiglu_gemm_applies()):
+                and self._swiglu_gemm_applies() and not self._six_bit_gate_up(q, s)):
             # prefill: gate and up in one launch that stores silu(gate) * up only (no fp16 [M, I] round trips)
             s, z, q = self._token_quant("mlp_mid", LinearFLH.forward_swiglu(self.gate_proj, self.up_proj, q, s))
             return x, self.down_proj(q, s, z, x_is_packed=True)

@@ -90,12 +90,25 @@ class W4A4LlamaModel(torch.nn.Module):
             x = fast_hadamard_transform(x, group_size=128, normalize=True)
         return x
 
+    def _rotary(self, positions, cache):
+        """cos / sin [T, head_dim] of `positions`.  With a static cache the table of all its slots is computed once and
+        the step's rows are gathered from it (two small launches instead of the dozen that build a table), the same
+        values either way."""
+        if cache is None:
+            return rotary_tables(positions, self.shape.head_dim, self.shape.rope_theta)
+        table = getattr(cache, "rotary_table", None)
+        if table is None:
+            table = rotary_tables(torch.arange(cache.max_len, device=positions.device), self.shape.head_dim,
+                                  self.shape.rope_theta)
+            cache.rotary_table = table
+        return table[0].index_select(0, positions), table[1].index_select(0, positions)
+
     def forward(self, input_ids, positions, cache=None, return_hidden=False):
         """input_ids [B, T] int64, positions [T] int64 (the same for every sequence of the batch).  cache: None (a
         fresh prefill without cache), or a StaticKVCache whose kv_len the caller has set to the number of slots
         attention may read (>= positions.max() + 1).  Returns logits [B, T, vocab] fp16 (or the final hidden state)."""
         x = self.embed(input_ids)
-        cos, sin = rotary_tables(positions, self.shape.head_dim, self.shape.rope_theta)
+        cos, sin = self._rotary(positions, cache)
         pending = None            # the last MLP output, added inside the next layer's first launch
         for i, layer in enumerate(self.layers):
             x, pending, _ = layer.forward_deferred(x, pending, cos, sin, cache.layer(i) if cache is not None else None,

@@ -285,6 +285,18 @@ int flh_decode_attention_f16(const flh_half* q, const flh_half* k_cache, const f
                              uint32_t B, uint32_t Hq, uint32_t Hkv, uint32_t head_dim, uint32_t kv_len, uint32_t max_len,
                              float scale, void* workspace, size_t workspace_bytes, void* stream);
 
+/* flh_decode_attention_f16 with the rotary embedding and the cache update of the step's new token inside, replacing
+ * flh_rope_kv_cache_f16 (T = 1) + flh_decode_attention_f16 by one pair of launches: q [B, Hq, d], k_new / v_new [B, Hkv, d]
+ * as the q / k / v GEMM wrote them (not rotated), cos / sin [d] of the new position, positions[0] (device int64) the
+ * cache slot the new token takes in every sequence (< kv_len, else the new token is ignored).  The rotated key and the
+ * value are written into k_cache / v_cache [B, Hkv, max_len, d] at that slot -- the same bytes flh_rope_kv_cache_f16 writes
+ * -- and attention runs over the first kv_len slots including it; q is left as it came.  Reference: apply_rotary_pos_emb +
+ * cache update + attention, flh/quantized_model/modeling_llama.py:403-460. */
+int flh_decode_attention_rope_f16(const flh_half* q, const flh_half* k_new, const flh_half* v_new, const flh_half* cos,
+                                  const flh_half* sin, const int64_t* positions, flh_half* k_cache, flh_half* v_cache,
+                                  flh_half* out, uint32_t B, uint32_t Hq, uint32_t Hkv, uint32_t head_dim, uint32_t kv_len,
+                                  uint32_t max_len, float scale, void* workspace, size_t workspace_bytes, void* stream);
+
 /* flh_decode_attention_f16 for callers that cannot allocate device memory and have no workspace to hand over -- code
  * under stream capture, tight serving loops, harnesses that forbid allocation.  No counterpart in the reference.  It
  * allocates nothing: the partial results go to a static device array of flh_decode_attention_static_scratch_bytes()

@@ -64,3 +64,57 @@ def test_decode_attention_argument_errors():
         _ops.decode_attention(q, k, k, 17)                             # kv_len beyond the cache
     with pytest.raises(RuntimeError):
         _ops.decode_attention(q, k, k, 8, workspace=torch.zeros(16, dtype=torch.uint8, device="cuda"))
+
+
+@pytest.mark.parametrize("b,hq,hkv,d,kv_len,max_len,slot", [(1, 32, 8, 128, 2048, 2048, 2047), (16, 32, 8, 128, 2048, 2048, 2047),
+                                                            (3, 32, 32, 128, 777, 1024, 776), (2, 8, 4, 64, 65, 128, 64),
+                                                            (2, 8, 1, 128, 1, 64, 0), (2, 16, 8, 64, 130, 256, 70),
+                                                            (2, 8, 8, 128, 200, 256, 63)])
+def test_rotary_and_cache_write_inside_attention_give_the_separate_launches_bits(b, hq, hkv, d, kv_len, max_len, slot):
+    """flh_decode_attention_rope_f16 against flh_rope_kv_cache_f16 followed by flh_decode_attention_f16 on copies of the
+    same cache: the same output, the same cache contents, bit for bit (slot at the end of the live range, at a chunk
+    boundary, in the middle -- an overwrite of an older position -- and slot 0 of an empty cache); q is left alone."""
+    from flh_amd import _ops
+    from flh_amd.quantized_model.decoder_layer import rotary_tables
+    gen = torch.Generator(device="cuda").manual_seed(kv_len + b + slot)
+    q = torch.randn(b, hq, d, device="cuda", generator=gen).half()
+    k_new = torch.randn(b, hkv, d, device="cuda", generator=gen).half()
+    v_new = torch.randn(b, hkv, d, device="cuda", generator=gen).half()
+    k = (torch.randn(b, hkv, max_len, d, device="cuda", generator=gen) * 0.5).half()
+    v = torch.randn(b, hkv, max_len, d, device="cuda", generator=gen).half()
+    k[:, :, kv_len:] = 100.0
+    v[:, :, kv_len:] = float("nan")
+    k[:, :, slot] = float("nan")                                       # what the slot held before must not be read
+    v[:, :, slot] = float("nan")
+    pos = torch.tensor([slot], device="cuda")
+    cos, sin = rotary_tables(pos, d, 500000.0)
+    print(f"case rotary decode attention b={b} hq={hq} hkv={hkv} d={d} kv_len={kv_len} slot={slot}", flush=True)
+    # separate launches
+    k1, v1, q1 = k.clone(), v.clone(), q.clone()
+    _ops.rope_kv_cache_(q1.view(b, 1, hq, d), k_new.view(b, 1, hkv, d), v_new.view(b, 1, hkv, d), cos, sin, pos, k1, v1)
+    want = _ops.decode_attention(q1, k1, v1, kv_len)
+    # one pair of launches
+    k2, v2, q2 = k.clone(), v.clone(), q.clone()
+    got = _ops.decode_attention_rope(q2, k_new, v_new, cos, sin, pos, k2, v2, kv_len)
+    assert torch.equal(q2, q)
+    assert torch.equal(got, want)
+    assert torch.equal(k2.view(torch.int16), k1.view(torch.int16)) and torch.equal(v2.view(torch.int16), v1.view(torch.int16))
+    ref = reference(q1, k1, v1, kv_len)
+    assert np.abs(got.cpu().numpy().astype(np.float64) - ref.astype(np.float64)).max() <= 2e-3 * max(1.0, np.abs(ref).max())
+
+
+def test_rotary_decode_attention_argument_errors():
+    from flh_amd import _ops
+    q = torch.zeros(1, 8, 128, device="cuda", dtype=torch.float16)
+    kn = torch.zeros(1, 2, 128, device="cuda", dtype=torch.float16)
+    k = torch.zeros(1, 2, 16, 128, device="cuda", dtype=torch.float16)
+    cs = torch.zeros(1, 128, device="cuda", dtype=torch.float16)
+    pos = torch.zeros(1, device="cuda", dtype=torch.int64)
+    with pytest.raises(RuntimeError):
+        _ops.decode_attention_rope(q, kn[:, :1].contiguous(), kn, cs, cs, pos, k, k.clone(), 4)
+    with pytest.raises(RuntimeError):
+        _ops.decode_attention_rope(q, kn, kn, cs[:, :64].contiguous(), cs, pos, k, k.clone(), 4)
+    with pytest.raises(RuntimeError):
+        _ops.decode_attention_rope(q, kn, kn, cs, cs, pos.int(), k, k.clone(), 4)
+    with pytest.raises(RuntimeError):
+        _ops.decode_attention_rope(q, kn, kn, cs, cs, pos, k, k.clone(), 17)

@@ -108,11 +108,13 @@ def test_token_configuration():
 
 
 def test_six_bit_layer_gives_the_same_bits():
-    w, plain = make(seed=9)
+    w, _ = make(seed=9)
+    plain = W4A4DecoderLayer.from_float(w, 4, 2, six_bit=False)
     six = W4A4DecoderLayer.from_float(w, 4, 2, six_bit=True)
     x = torch.randn(1, 300, 512, generator=torch.Generator().manual_seed(10)).half().cuda()
     cos, sin = rotary_tables(torch.arange(300, device="cuda"), 128)
     a, (ka, va) = plain(x, cos, sin)
     b, (kb, vb) = six(x, cos, sin)
     assert six.q_proj._w6 is not None and six.down_proj._w6 is not None     # the 6-bit path really ran
+    assert plain.q_proj._w6 is None and plain.down_proj._w6 is None
     assert torch.equal(a, b) and torch.equal(ka, kb) and torch.equal(va, vb)

@@ -223,7 +223,9 @@ def test_linear_flh_six_bit_switch_gives_the_same_bits(group):
     layer = LinearFLH.from_float(lin, weight_group_size=group, in_group_size=128, no_hadamard=True)
     x = (torch.randn(m, k, device="cuda") * 2).half()
     q, s = flh_amd._CUDA.rotate_and_quantize_i4(x, hadamard=False)             # one scale per token
+    layer.six_bit = False
     want = layer(q, s, x_is_packed=True)
+    assert layer._w6 is None
     layer.six_bit = True
     got = layer(q, s, x_is_packed=True)
     assert layer._w6 is not None and torch.equal(got, want)
@@ -243,9 +245,13 @@ def test_six_bit_quantiser_feeds_linear_flh(had):
     s4, z4, q4 = ActQuantizerGS(group_size=128, use_hadamard=had)(x)
     s6, z6, q6 = ActQuantizerGS(group_size=128, use_hadamard=had, six_bit=True)(x)
     assert torch.equal(s4, s6) and q6.shape == (2, m // 2, k // 128 * 96)
+    layer.six_bit = False
     want = layer(q4, s4, z4, x_is_packed=True)
+    assert layer._w6 is None
     got = layer(q6, s6, z6, x_is_packed=True)
     assert got.shape == want.shape and torch.equal(got, want)
+    layer.six_bit = None           # the default: group-scaled weights take the 6-bit instruction from 256 rows on
+    assert torch.equal(layer(q4, s4, z4, x_is_packed=True), want)
 
 
 @pytest.mark.parametrize("tokens,group", [(1, 0), (2, 128), (7, 0), (7, 128)])
@@ -293,7 +299,10 @@ def test_forward_many_on_the_six_bit_path(group):
         s, z, q = ActQuantizerGS(group_size=128, use_hadamard=True)(x)
     else:
         q, s = flh_amd._CUDA.rotate_and_quantize_i4(x, hadamard="exact")
+    for layer in layers:
+        layer.six_bit = False
     want = LinearFLH.forward_many(layers, q, s)
+    assert all(layer._w6 is None for layer in layers)
     for layer in layers:
         layer.six_bit = True
     got = LinearFLH.forward_many(layers, q, s)
