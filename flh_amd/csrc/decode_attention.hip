@@ -43,10 +43,10 @@ __global__ __launch_bounds__(kAttnThreads) void decode_attention_partial_kernel(
     const long long* __restrict__ positions) {
   static_assert(D == 128 || D == 64, "head dimension");
   static_assert(CHUNK == 64, "one key per lane in the softmax step");
-  constexpr int TPK = kAttnThreads / CHUNK;            // threads per key: 4
-  constexpr int CPT = D / TPK;                         // channels per thread in the score step: 32 (16)
-  constexpr int RPW = CHUNK / (kAttnThreads / 64);     // value rows per wave: 16
-  __shared__ float qs[REP * D];                        // the query heads as float
+  static_assert(REP <= 16, "the heads of a key / value head are the columns of one matrix tile");
+  constexpr int KS = D / 32;                           // matrix steps over the channels
+  constexpr int RPW = CHUNK / (kAttnThreads / 64);     // keys / value rows per wave: 16
+  __shared__ __align__(16) _Float16 qs[REP * D];       // the query heads
   __shared__ float sc[REP][CHUNK];                     // scores, then probabilities
   __shared__ float red[kAttnThreads / 64][REP * D];    // the waves' weighted values
   const int tid = threadIdx.x, lane = tid & 63;
@@ -58,86 +58,82 @@ __global__ __launch_bounds__(kAttnThreads) void decode_attention_partial_kernel(
     const long long pos = positions[0];
     if (pos >= 0 && pos < (long long)kv_len) slot = (uint32_t)pos;
   }
-  const __half* qh = q + (size_t)bh * REP * D;         // q [B, Hq, D]: the REP heads of this kv head are adjacent
+  const _Float16* qf = (const _Float16*)q + (size_t)bh * REP * D;   // q [B, Hq, D]: the REP heads of this kv head are adjacent
   for (int i = tid; i < REP * D; i += kAttnThreads) {
     if constexpr (ROPE) {
+      const _Float16 *cf = (const _Float16*)cos, *sf = (const _Float16*)sin;
       const int d = i % D;
-      const _Float16 *qf = (const _Float16*)qh, *cf = (const _Float16*)cos, *sf = (const _Float16*)sin;
-      qs[i] = (float)rope_value(qf[i], qf[i ^ (D / 2)], cf[d], sf[d], d < D / 2);
+      qs[i] = rope_value(qf[i], qf[i ^ (D / 2)], cf[d], sf[d], d < D / 2);
     } else {
-      qs[i] = __half2float(qh[i]);
+      qs[i] = qf[i];
     }
   }
 
-  // scores: thread (key, part) takes CPT channels of its key
-  const int key = tid / TPK, part = tid % TPK;
-  const uint32_t t = t0 + key;
+  // Scores on the matrix cores: wave w owns the keys 16 w .. 16 w + 15 as the rows of a 16 x 16 tile whose columns are
+  // the query heads; a lane holds eight consecutive channels (block `kb` of the step's 32) of key row `krow`.
+  const int krow = lane & 15, kb = lane >> 4;
+  const uint32_t t = t0 + wave * RPW + krow;
   const bool live = t < kv_len;
-  float kv[CPT];
+  h8 ka[KS];
   if (ROPE && t == slot) {                             // the new key: rotate it, keep it, and store it in its slot
     const __half* src = k_new + (size_t)bh * D;
-    const int c0 = part * CPT, p0 = c0 ^ (D / 2);
-    __half* dst = k_cache + ((size_t)bh * max_len + t) * D + c0;
+    __half* dst = k_cache + ((size_t)bh * max_len + t) * D;
 #pragma unroll
-    for (int c8 = 0; c8 < CPT / 8; ++c8) {
-      const h8 x = *(const h8*)(src + c0 + c8 * 8), xp = *(const h8*)(src + p0 + c8 * 8);
-      const h8 cc = *(const h8*)(cos + c0 + c8 * 8), ss = *(const h8*)(sin + c0 + c8 * 8);
+    for (int ks = 0; ks < KS; ++ks) {
+      const int c0 = ks * 32 + kb * 8, p0 = c0 ^ (D / 2);
+      const h8 x = *(const h8*)(src + c0), xp = *(const h8*)(src + p0);
+      const h8 cc = *(const h8*)(cos + c0), ss = *(const h8*)(sin + c0);
       h8 y;
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        y[e] = rope_value(x[e], xp[e], cc[e], ss[e], c0 < D / 2);
-        kv[c8 * 8 + e] = (float)y[e];
-      }
-      *(h8*)(dst + c8 * 8) = y;
+      for (int e = 0; e < 8; ++e) y[e] = rope_value(x[e], xp[e], cc[e], ss[e], c0 < D / 2);
+      ka[ks] = y;
+      *(h8*)(dst + c0) = y;
     }
   } else {
-    const __half* kr = k_cache + ((size_t)bh * max_len + (live ? t : 0)) * D + part * CPT;
+    const __half* kr = k_cache + ((size_t)bh * max_len + (live ? t : 0)) * D + kb * 8;
 #pragma unroll
-    for (int c8 = 0; c8 < CPT / 8; ++c8) {
-      const h8 v = *(const h8*)(kr + c8 * 8);
-#pragma unroll
-      for (int e = 0; e < 8; ++e) kv[c8 * 8 + e] = (float)v[e];
-    }
+    for (int ks = 0; ks < KS; ++ks) ka[ks] = *(const h8*)(kr + ks * 32);
   }
   // Values: wave w takes rows 16 w .. 16 w + 15 of the chunk, a lane one channel pair (one channel for D = 64) of
-  // each; requested now, the loads travel while the scores and the softmax pieces are computed.
+  // each; requested now, the loads travel while the scores and the softmax pieces are computed.  Rows past the live
+  // range read the last live row again (any valid address) and are zeroed: their probability is zero, but 0 x NaN is not.
   const uint32_t n_live = kv_len > t0 ? min((uint32_t)CHUNK, kv_len - t0) : 0u;
-  __half* vr = v_cache + ((size_t)bh * max_len + t0 + wave * RPW) * D;
+  __half* vbase = v_cache + ((size_t)bh * max_len + t0) * D;
   float vv0[RPW], vv1[D == 128 ? RPW : 1];
 #pragma unroll
   for (int i = 0; i < RPW; ++i) {
     const uint32_t row = wave * RPW + i;               // wave-uniform
     const bool fresh = ROPE && t0 + row == slot;
+    const bool have = row < n_live;
+    const __half* src = fresh ? v_new + (size_t)bh * D : vbase + (size_t)(have ? row : (n_live ? n_live - 1 : 0)) * D;
     if constexpr (D == 128) {
-      h2 v = {(_Float16)0.f, (_Float16)0.f};
-      if (fresh) {
-        v = *(const h2*)(v_new + (size_t)bh * D + 2 * lane);
-        *(h2*)(vr + (size_t)i * D + 2 * lane) = v;
-      } else if (row < n_live) {
-        v = *(const h2*)(vr + (size_t)i * D + 2 * lane);
-      }
-      vv0[i] = (float)v[0];
-      vv1[i] = (float)v[1];
+      h2 v = *(const h2*)(src + 2 * lane);
+      if (fresh) *(h2*)(vbase + (size_t)row * D + 2 * lane) = v;
+      vv0[i] = have ? (float)v[0] : 0.f;
+      vv1[i] = have ? (float)v[1] : 0.f;
     } else {
-      __half v = __float2half(0.f);
-      if (fresh) {
-        v = v_new[(size_t)bh * D + lane];
-        vr[(size_t)i * D + lane] = v;
-      } else if (row < n_live) {
-        v = vr[(size_t)i * D + lane];
-      }
-      vv0[i] = __half2float(v);
+      const __half v = src[lane];
+      if (fresh) vbase[(size_t)row * D + lane] = v;
+      vv0[i] = have ? __half2float(v) : 0.f;
     }
   }
   __syncthreads();                                     // the queries are in LDS
+  {
+    v4f acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-  for (int h = 0; h < REP; ++h) {
-    float s = 0.f;
+    for (int ks = 0; ks < KS; ++ks) {
+      h8 qb = {0, 0, 0, 0, 0, 0, 0, 0};
+      if (krow < REP) qb = *(const h8*)(qs + krow * D + ks * 32 + kb * 8);   // column `krow` of the tile: head krow
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka[ks], qb, acc, 0, 0, 0);
+    }
+    // acc[i]: key 16 w + 4 kb + i, head krow
+    if (krow < REP) {
 #pragma unroll
-    for (int c = 0; c < CPT; ++c) s = __builtin_fmaf(kv[c], qs[h * D + part * CPT + c], s);
-    s += dpp_f<kDppQuadXor1>(s);                       // the four threads of a key are one quad
-    s += dpp_f<kDppQuadXor2>(s);
-    if (part == 0) sc[h][key] = live ? s * scale : -INFINITY;
+      for (int i = 0; i < 4; ++i) {
+        const uint32_t key = wave * RPW + 4 * kb + i;
+        sc[krow][key] = t0 + key < kv_len ? acc[i] * scale : -INFINITY;
+      }
+    }
   }
   __syncthreads();
 
