@@ -35,5 +35,11 @@ than "retyping the formula" fixes each function) is listed per module; the summa
                    attention, pinned by special cases (tests/test_oracle_layer.py).
 * ``gptq``      -- GPTQ in the rotated basis in its elimination form, pinned by closed forms and properties
                    (tests/test_oracle_gptq.py).
+
+Parity unpinned (no vector of the reference can exist here, and no closed form decides the open choice):
+``gemm.gemm_i4_dequant`` with group scales beyond rtol 1e-3 / atol 1e-2 (whether the reference's compiler fuses the
+multiply-add of the fold cannot be observed); ``quant.kernel_had_and_quant`` on random data (CUDA-only arithmetic:
+fp16 butterflies and the ``s <= 1e-6`` rule are restated from the kernel's text, pinned on integer and closed-form rows
+only); ``gptq.gptq`` beyond the properties above (the reference's implementation is CUDA-bound and was read, not run).
 """
 from . import pack, hadamard, quant, gemm, linear  # noqa: F401
