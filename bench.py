@@ -196,8 +196,10 @@ def main():
         return ms, {k: float(np.median(v)) for k, v in per.items()}
 
     other_form = "seven" if args.launches == "layer" else "layer"
+    # the other form first: the first few hundred launches of a process run below the steady rate (clocks and caches
+    # settle for longer than a handful of warm-up steps), which would otherwise be charged to whichever form is timed first
     ms_other, med_other = run_form(other_form)
-    ms_per_step, med = run_form(args.launches)      # the headline: timed last, on a warm device
+    ms_per_step, med = run_form(args.launches)      # the headline: --warmup untimed steps, then exactly --steps timed ones
     step = make_step("seven")
 
     # The same step with the weights of projections that share an input stored concatenated ([q; k; v] and
