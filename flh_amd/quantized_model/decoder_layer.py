@@ -278,6 +278,24 @@ class W4A4DecoderLayer(torch.nn.Module):
                                               vs.view(b, t, self.num_kv_heads, self.head_dim), cos, sin, positions)
             cache = kv_cache
             qs = qs.transpose(1, 2)
+        elif (self.fused and x.is_cuda and self.head_dim % 16 == 0 and cos.dtype == torch.float16
+              and cos.shape == (t, self.head_dim)):
+            # a growing pair of tensors as cache: the same rotary / cache-write launch on freshly allocated keys / values
+            # (the bits of the tensor expression of the branch below, in one launch instead of a dozen)
+            past = 0 if kv_cache is None else kv_cache[0].size(2)
+            keys = torch.empty(b, self.num_kv_heads, past + t, self.head_dim, dtype=qs.dtype, device=x.device)
+            values = torch.empty_like(keys)
+            if past:
+                keys[:, :, :past] = kv_cache[0]
+                values[:, :, :past] = kv_cache[1]
+            slots = torch.arange(past, past + t, device=x.device)
+            qs = qs.view(b, t, self.num_heads, self.head_dim)
+            _ops().rope_kv_cache_(qs, ks.view(b, t, self.num_kv_heads, self.head_dim),
+                                  vs.view(b, t, self.num_kv_heads, self.head_dim), cos.contiguous(), sin.contiguous(),
+                                  slots, keys, values)
+            qs = qs.transpose(1, 2)
+            ks, vs = keys, values
+            cache = (ks, vs)
         else:
             qs = qs.view(b, t, self.num_heads, self.head_dim).transpose(1, 2)
             ks = ks.view(b, t, self.num_kv_heads, self.head_dim).transpose(1, 2)
