@@ -692,8 +692,14 @@ def main():
             def linears_only():
                 for layer in model5.layers:
                     nw = layer._norm_weight16("input_layernorm", layer.input_layernorm)
-                    _, q5, s5 = ops.add_rmsnorm_rotate_and_quantize_i4(xb5, xb5b, nw, 1e-5)
-                    LinearFLH.forward_many([layer.q_proj, layer.k_proj, layer.v_proj], q5, s5)
+                    if batch <= 2:      # residual addition, norm, quantiser and q / k / v in one launch
+                        qkv = [layer.q_proj, layer.k_proj, layer.v_proj]
+                        ops.rmsnorm_rotate_quantize_gemm_i4_multi(
+                            xb5, xb5b, nw, 1e-5, [l.w_packed.view(l.out_features, l.in_features // 2) for l in qkv],
+                            [l.w_scale.view(l.out_features, -1) for l in qkv])
+                    else:
+                        _, q5, s5 = ops.add_rmsnorm_rotate_and_quantize_i4(xb5, xb5b, nw, 1e-5)
+                        LinearFLH.forward_many([layer.q_proj, layer.k_proj, layer.v_proj], q5, s5)
                     if batch <= 2:
                         layer.o_proj.forward_online(xb5, hadamard="exact")
                     else:

@@ -223,6 +223,44 @@ def rotate_quantize_gemm_i4_multi(x, Bs, B_scales):
     return Ds
 
 
+def rmsnorm_rotate_quantize_gemm_i4_multi(x, add, weight, eps, Bs, B_scales):
+    """rotate_quantize_gemm_i4_multi on RMSNorm(x [+ add]) in one launch: x (and add, or None) [M, 4096] fp16 with M <= 4,
+    weight [4096] fp16 or None -> (x + add [M, 4096] fp16 or None, [fp16 [M, N_s] ...]); the outputs are those of
+    [add_]rmsnorm_rotate_and_quantize_i4 followed by gemm_i4_dequant_multi, bit for bit."""
+    import ctypes
+    _check(len(Bs) == len(B_scales) and 1 <= len(Bs) <= 4, "one to four weight matrices, one scale tensor each")
+    _check(x.is_cuda and x.dtype == torch.float16 and x.dim() == 2 and x.is_contiguous(),
+           "x must be a contiguous 2D float16 CUDA tensor")
+    M, K = x.shape
+    _check(M <= ROTATE_GEMM_MAX_TOKENS, "at most 4 tokens")
+    _check(K in ROTATE_GEMM_WIDTHS, "K must be 4096")
+    if add is not None:
+        _check(add.is_cuda and add.dtype == torch.float16 and add.shape == x.shape and add.is_contiguous()
+               and add.device == x.device, "add must be a contiguous float16 CUDA tensor of x's shape")
+    if weight is not None:
+        _check(weight.is_cuda and weight.dtype == torch.float16 and weight.is_contiguous() and weight.numel() == K
+               and weight.device == x.device, "weight must be a contiguous float16 CUDA tensor of K values")
+    for B, S in zip(Bs, B_scales):
+        _check(B.is_cuda and S.is_cuda and B.device == x.device and S.device == x.device, "tensors must be on one device")
+        _check(B.dtype == torch.uint8 and B.dim() == 2 and B.is_contiguous() and B.size(1) * 2 == K,
+               "B must be a contiguous uint8 [N, K/2] tensor")
+        _check(S.dtype == torch.float16 and S.is_contiguous() and S.dim() == 2 and S.size(0) == B.size(0)
+               and S.size(1) in (1, K // 128) and S.size(1) == B_scales[0].size(1),
+               "B_scale must be a contiguous float16 [N, 1] or [N, K/128] tensor, the same width for every matrix")
+        _check(B.size(0) > 0, "empty weight matrix")
+    total = torch.empty_like(x) if add is not None else None
+    Ds = [torch.empty((M, B.size(0)), dtype=torch.float16, device=x.device) for B in Bs]
+    if M:
+        n = len(Bs)
+        ptrs = lambda ts: (ctypes.c_void_p * n)(*[t.data_ptr() for t in ts])
+        sizes = (ctypes.c_size_t * n)(*[B.size(0) for B in Bs])
+        _run("flh_rmsnorm_rotate_quant_gemm_i4_o16_multi", x.device, x.data_ptr(),
+             add.data_ptr() if add is not None else None, total.data_ptr() if total is not None else None,
+             weight.data_ptr() if weight is not None else None, float(eps), n, ptrs(Bs), ptrs(B_scales), ptrs(Ds), sizes,
+             M, K, B_scales[0].size(1), _stream(x))
+    return total, Ds
+
+
 def gemm_set_tuning(tile=0, k_split=0):
     """Test / tuning hook: force the GEMM tile (64, 128, 256) and in-workgroup K split (1, 2, 4); 0 = automatic."""
     _lib.check(_lib.load().flh_gemm_set_tuning(int(tile), int(k_split)))

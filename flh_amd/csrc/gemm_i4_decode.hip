@@ -202,9 +202,21 @@ int launch_decode(const GemmArgs& a, hipStream_t stream) {
 // codes and scales are the same bits -- while the weights are still on their way from HBM.  The rotation is
 // repeated by every workgroup (about a microsecond per token); what it saves is a whole launch in front of the
 // GEMM, which is worth more than that for one or two tokens and outputs up to about 12 K channels.
-template <int EPI>
+//
+// NORM / ADD: the tokens are RMS-normalised first (NORM), after a residual addition x + add (ADD) -- the prologues of
+// flh_rmsnorm_rotate_quant_i4 / flh_add_rmsnorm_rotate_quant_i4 with the same roundings, so again the same bits as the
+// separate launches.  Every workgroup forms the sum for itself; workgroup 0 stores it (the new residual stream).
+struct DecodePrologue {
+  const __half* rms_weight;   // NORM: null = no weight
+  float eps;
+  const __half* add;          // ADD
+  __half* sum_out;            // ADD
+};
+
+template <int EPI, bool NORM = false, bool ADD = false>
 __global__ __launch_bounds__(kWaves * 64) void rotate_gemm_i4_decode_kernel(const __half* __restrict__ x,
-                                                                            const GemmArgs p, float norm) {
+                                                                            const GemmArgs p, float norm,
+                                                                            const DecodePrologue pro) {
   constexpr int K = 4096, Kb = K / 2, KT = K / 128, ND = KT / 2, NDW = ND / kWaves;
   constexpr int ROW = Kb + 16;                 // code rows 16 bytes apart in the banks
   constexpr int TILES = EPI == kGroupScale ? KT : 2 * kWaves;   // at least the 16 KB the rotation stages in
@@ -234,8 +246,14 @@ __global__ __launch_bounds__(kWaves * 64) void rotate_gemm_i4_decode_kernel(cons
       sB[g * 16 + row] = n0 + row < w.N ? __half2float(w.Bs[(size_t)(n0 + row) * KT + g]) : 0.f;
     }
   }
-  for (int row = 0; row < p.M; ++row)
-    rotate_quant_row_8waves(x + (size_t)row * K, (float*)red, sA, codes + row * ROW, tok + row, norm, wave);
+  for (int row = 0; row < p.M; ++row) {
+    if constexpr (NORM || ADD)
+      rotate_quant_row_8waves<NORM, ADD>(x + (size_t)row * K, (float*)red, sA, codes + row * ROW, tok + row, norm, wave,
+                                         pro.rms_weight, pro.eps, ADD ? pro.add + (size_t)row * K : nullptr,
+                                         ADD && blockIdx.x == 0 ? pro.sum_out + (size_t)row * K : nullptr);
+    else
+      rotate_quant_row_8waves(x + (size_t)row * K, (float*)red, sA, codes + row * ROW, tok + row, norm, wave);
+  }
   __syncthreads();
   if (tid < 16) sA[tid] = tid < p.M ? __half2float(tok[tid]) : 0.f;
 
@@ -263,14 +281,21 @@ __global__ __launch_bounds__(kWaves * 64) void rotate_gemm_i4_decode_kernel(cons
 }
 
 template <int EPI>
-int launch_rotate_decode(const __half* x, const GemmArgs& a, hipStream_t stream) {
+int launch_rotate_decode(const __half* x, const GemmArgs& a, hipStream_t stream, const DecodePrologue* pro = nullptr) {
   constexpr int K = 4096, KT = K / 128;
   constexpr size_t smem = (size_t)(EPI == kGroupScale ? KT : 2 * kWaves) * 1024 + KT * 64 + 64 +
                           kRotateGemmMaxTokens * (K / 2 + 16) + 32;
   static_assert(smem <= 64 * 1024, "fits the default dynamic LDS limit");
   GemmArgs g = a;
   const int blocks = decode_blocks(g);
-  hipLaunchKernelGGL((rotate_gemm_i4_decode_kernel<EPI>), dim3(blocks), dim3(kWaves * 64), smem, stream, x, g, 1.0f / 64.0f);
+  const dim3 grid(blocks), block(kWaves * 64);
+  const DecodePrologue none{nullptr, 0.f, nullptr, nullptr};
+  if (!pro)
+    hipLaunchKernelGGL((rotate_gemm_i4_decode_kernel<EPI>), grid, block, smem, stream, x, g, 1.0f / 64.0f, none);
+  else if (pro->add)
+    hipLaunchKernelGGL((rotate_gemm_i4_decode_kernel<EPI, true, true>), grid, block, smem, stream, x, g, 1.0f / 64.0f, *pro);
+  else
+    hipLaunchKernelGGL((rotate_gemm_i4_decode_kernel<EPI, true, false>), grid, block, smem, stream, x, g, 1.0f / 64.0f, *pro);
   return check_launch("rotate_gemm_i4_decode");
 }
 
@@ -297,30 +322,31 @@ int gemm_decode_dispatch(const GemmArgs& a, int epi, hipStream_t stream) {
 
 }  // namespace flh
 
-extern "C" int flh_rotate_quant_gemm_i4_o16_multi(const flh_half* x, int count, const uint8_t* const* B,
-                                                  const flh_half* const* b_scale, flh_half* const* D, const size_t* N,
-                                                  size_t M, size_t K, int b_cols, void* stream) {
+namespace {
+int rotate_gemm_checked(const char* who, const flh_half* x, const flh::DecodePrologue* pro, int count,
+                        const uint8_t* const* B, const flh_half* const* b_scale, flh_half* const* D, const size_t* N,
+                        size_t M, size_t K, int b_cols, void* stream) {
   using namespace flh;
   if (count < 1 || count > kMaxGemmSegments)
-    return fail(FLH_EINVAL, "rotate_quant_gemm: count = %d, must be 1 .. %d", count, kMaxGemmSegments);
-  if (!B || !b_scale || !D || !N) return fail(FLH_EINVAL, "rotate_quant_gemm: null array");
+    return fail(FLH_EINVAL, "%s: count = %d, must be 1 .. %d", who, count, kMaxGemmSegments);
+  if (!B || !b_scale || !D || !N) return fail(FLH_EINVAL, "%s: null array", who);
   if (M == 0) return FLH_OK;
-  if (!x) return fail(FLH_EINVAL, "rotate_quant_gemm: null pointer");
-  if (misaligned16(x)) return fail(FLH_EINVAL, "rotate_quant_gemm: x must be 16-byte aligned");
+  if (!x) return fail(FLH_EINVAL, "%s: null pointer", who);
+  if (misaligned16(x)) return fail(FLH_EINVAL, "%s: x must be 16-byte aligned", who);
   if (M > (size_t)kRotateGemmMaxTokens)
-    return fail(FLH_EINVAL, "rotate_quant_gemm: M = %zu, at most %d tokens (more tokens quantise once, in their own launch)",
-                M, kRotateGemmMaxTokens);
-  if (K != 4096) return fail(FLH_EINVAL, "rotate_quant_gemm: K = %zu is not supported (4096)", K);
+    return fail(FLH_EINVAL, "%s: M = %zu, at most %d tokens (more tokens quantise once, in their own launch)", who, M,
+                kRotateGemmMaxTokens);
+  if (K != 4096) return fail(FLH_EINVAL, "%s: K = %zu is not supported (4096)", who, K);
   if (b_cols != 1 && (size_t)b_cols != K / 128)
-    return fail(FLH_EINVAL, "rotate_quant_gemm: weight scale columns (%d) must be 1 or K / 128 = %zu", b_cols, K / 128);
+    return fail(FLH_EINVAL, "%s: weight scale columns (%d) must be 1 or K / 128 = %zu", who, b_cols, K / 128);
   size_t n_all = 0;
   for (int s = 0; s < count; ++s) {
-    if (N[s] == 0) return fail(FLH_EINVAL, "rotate_quant_gemm: N[%d] = 0", s);
-    if (!B[s] || !b_scale[s] || !D[s]) return fail(FLH_EINVAL, "rotate_quant_gemm: null pointer");
-    if (misaligned16(B[s], D[s])) return fail(FLH_EINVAL, "rotate_quant_gemm: B and D must be 16-byte aligned");
+    if (N[s] == 0) return fail(FLH_EINVAL, "%s: N[%d] = 0", who, s);
+    if (!B[s] || !b_scale[s] || !D[s]) return fail(FLH_EINVAL, "%s: null pointer", who);
+    if (misaligned16(B[s], D[s])) return fail(FLH_EINVAL, "%s: B and D must be 16-byte aligned", who);
     n_all += N[s];
   }
-  if (n_all > (1u << 30)) return fail(FLH_EINVAL, "rotate_quant_gemm: N too large");
+  if (n_all > (1u << 30)) return fail(FLH_EINVAL, "%s: N too large", who);
   GemmArgs g{nullptr, B[0], nullptr, (const __half*)b_scale[0], D[0], (int)M, (int)N[0], (int)K, 1, b_cols, 0, 0, 0};
   g.n_seg = count;
   for (int s = 1; s < count; ++s) {
@@ -329,8 +355,32 @@ extern "C" int flh_rotate_quant_gemm_i4_o16_multi(const flh_half* x, int count, 
     g.seg_D[s] = D[s];
     g.seg_N[s] = (int)N[s];
   }
-  return b_cols == 1 ? launch_rotate_decode<kRowScale>((const __half*)x, g, (hipStream_t)stream)
-                     : launch_rotate_decode<kGroupScale>((const __half*)x, g, (hipStream_t)stream);
+  return b_cols == 1 ? launch_rotate_decode<kRowScale>((const __half*)x, g, (hipStream_t)stream, pro)
+                     : launch_rotate_decode<kGroupScale>((const __half*)x, g, (hipStream_t)stream, pro);
+}
+}  // namespace
+
+extern "C" int flh_rotate_quant_gemm_i4_o16_multi(const flh_half* x, int count, const uint8_t* const* B,
+                                                  const flh_half* const* b_scale, flh_half* const* D, const size_t* N,
+                                                  size_t M, size_t K, int b_cols, void* stream) {
+  return rotate_gemm_checked("rotate_quant_gemm", x, nullptr, count, B, b_scale, D, N, M, K, b_cols, stream);
+}
+
+extern "C" int flh_rmsnorm_rotate_quant_gemm_i4_o16_multi(const flh_half* x, const flh_half* add, flh_half* sum_out,
+                                                          const flh_half* weight, float eps, int count,
+                                                          const uint8_t* const* B, const flh_half* const* b_scale,
+                                                          flh_half* const* D, const size_t* N, size_t M, size_t K,
+                                                          int b_cols, void* stream) {
+  using namespace flh;
+  const char* who = "rmsnorm_rotate_quant_gemm";
+  if (!(eps >= 0.f)) return fail(FLH_EINVAL, "%s: eps must not be negative", who);
+  if ((add == nullptr) != (sum_out == nullptr)) return fail(FLH_EINVAL, "%s: add and sum_out come together or not at all", who);
+  if (add && (misaligned16(add, sum_out))) return fail(FLH_EINVAL, "%s: add and sum_out must be 16-byte aligned", who);
+  if (weight && misaligned16(weight)) return fail(FLH_EINVAL, "%s: weight must be 16-byte aligned", who);
+  if (sum_out && ((const void*)sum_out == (const void*)x || (const void*)sum_out == (const void*)add))
+    return fail(FLH_EINVAL, "%s: sum_out must not be x or add", who);
+  const DecodePrologue pro{(const __half*)weight, eps, (const __half*)add, (__half*)sum_out};
+  return rotate_gemm_checked(who, x, &pro, count, B, b_scale, D, N, M, K, b_cols, stream);
 }
 
 extern "C" int flh_rotate_quant_gemm_i4_o16(const flh_half* x, const uint8_t* B, const flh_half* b_scale, flh_half* D,

@@ -262,7 +262,7 @@ __device__ __forceinline__ void rotate_quant_row_8waves(const __half* __restrict
   v4i raw = *(const v4i*)(x_row + wave * 512 + c * 8);
   if constexpr (ADD) {
     raw = add_h8(raw, *(const v4i*)(add_row + wave * 512 + c * 8));
-    *(v4i*)(sum_row + wave * 512 + c * 8) = raw;
+    if (sum_row) *(v4i*)(sum_row + wave * 512 + c * 8) = raw;    // (null: another workgroup stores the same sum)
   }
   if constexpr (RMS) {
     float ss = 0.f;

@@ -253,9 +253,21 @@ class W4A4DecoderLayer(torch.nn.Module):
     def _attention(self, x, add, cos, sin, kv_cache=None, positions=None):
         """attention() on the residual stream x + add (add may be None); returns that sum as well."""
         b, t, _ = x.shape
-        x, s, z, q = self._residual_norm_quant("attn_in", self.input_layernorm, "input_layernorm", self.attn_quantizer1,
-                                               x, add)
-        qs, ks, vs = self._project([self.q_proj, self.k_proj, self.v_proj], q, s, z)
+        if (self.activation == "token" and self.fused and self.record is None and b * t <= 2 and self.hidden_size == 4096
+                and self._online_qkv_applies()):
+            # decode: residual addition, norm, rotation, quantiser and the three projections in one launch
+            layers = [self.q_proj, self.k_proj, self.v_proj]
+            total, (qs, ks, vs) = _ops().rmsnorm_rotate_quantize_gemm_i4_multi(
+                x.reshape(b * t, -1).contiguous(), None if add is None else add.reshape(b * t, -1).contiguous(),
+                self._norm_weight16("input_layernorm", self.input_layernorm), self.input_layernorm.eps,
+                [l.w_packed.view(l.out_features, l.in_features // 2) for l in layers],
+                [l.w_scale.view(l.out_features, -1) for l in layers])
+            if total is not None:
+                x = total.view(x.shape)
+        else:
+            x, s, z, q = self._residual_norm_quant("attn_in", self.input_layernorm, "input_layernorm",
+                                                   self.attn_quantizer1, x, add)
+            qs, ks, vs = self._project([self.q_proj, self.k_proj, self.v_proj], q, s, z)
         self._tap("q_proj", qs), self._tap("k_proj", ks), self._tap("v_proj", vs)
         static = isinstance(kv_cache, StaticKVCache._Layer)
         out = None
@@ -324,6 +336,15 @@ class W4A4DecoderLayer(torch.nn.Module):
         y = self.o_proj(q, s, z, x_is_packed=True)
         self._tap("o_proj", y)
         return x, y, cache
+
+    def _online_qkv_applies(self):
+        """q / k / v in the layout the decode GEMM with its own norm + quantiser takes: no bias, one scale per channel or
+        per group of 128, the same for all three."""
+        cols = {l.w_scale.view(l.out_features, -1).size(1) for l in (self.q_proj, self.k_proj, self.v_proj)}
+        if any(l.bias is not None for l in (self.q_proj, self.k_proj, self.v_proj)) or len(cols) != 1:
+            return False
+        c = cols.pop()
+        return c == 1 or (c == self.hidden_size // 128 and self.q_proj.weight_group_size == 128)
 
     def _swiglu_gemm_applies(self):
         g = self.gate_proj

@@ -100,6 +100,16 @@ int flh_rotate_quant_gemm_i4_o16_multi(const flh_half* x, int count, const uint8
                                        const flh_half* const* b_scale, flh_half* const* D, const size_t* N, size_t M,
                                        size_t K, int b_cols, void* stream);
 
+/* flh_rotate_quant_gemm_i4_o16_multi with the prologues of flh_rmsnorm_rotate_quant_i4 / flh_add_rmsnorm_rotate_quant_i4 in
+ * front of the rotation, still one launch: the tokens are RMS-normalised (weight [K] fp16 or null, eps), after the
+ * residual addition fp16(x + add) when add / sum_out [M, K] are given (both or neither; sum_out receives the sum and
+ * overlaps neither input).  M <= 4, K = 4096.  A decode step's "residual + attention output -> norm -> quantiser ->
+ * q / k / v" (flh/quantized_model/modeling_llama.py:389-393, 600-618) as one launch; same bits as the separate launches. */
+int flh_rmsnorm_rotate_quant_gemm_i4_o16_multi(const flh_half* x, const flh_half* add, flh_half* sum_out,
+                                               const flh_half* weight, float eps, int count, const uint8_t* const* B,
+                                               const flh_half* const* b_scale, flh_half* const* D, const size_t* N, size_t M,
+                                               size_t K, int b_cols, void* stream);
+
 /* Test and tuning hook (no counterpart in the reference): overrides, process-wide, the tile (64, 128 or 256 rows;
  * 0 = automatic) and the split of K inside a workgroup (1, 2 or 4; 0 = automatic) that flh_gemm_i4_o16 and
  * flh_gemm_f6_o16 would choose from the shape.  Every variant gives the same bits; the tests use this to reach

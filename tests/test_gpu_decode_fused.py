@@ -95,3 +95,40 @@ def test_argument_errors(ops):
     with pytest.raises(RuntimeError):
         ops.rotate_quantize_gemm_i4(torch.zeros(1, 4096, dtype=torch.float16, device="cuda"), wd, sd.repeat(1, 3))
     assert ops.rotate_quantize_gemm_i4(torch.zeros(0, 4096, dtype=torch.float16, device="cuda"), wd, sd).shape == (0, 32)
+
+
+@pytest.mark.parametrize("m", [1, 2, 4])
+@pytest.mark.parametrize("grouped", [False, True])
+@pytest.mark.parametrize("with_add,with_weight", [(False, True), (True, True), (True, False)])
+def test_norm_and_residual_prologue_equals_the_separate_launches(ops, m, grouped, with_add, with_weight):
+    """RMSNorm (and the residual addition in front of it) inside the decode GEMM: the sum, and every output, bit for bit
+    those of [add_]rmsnorm_rotate_and_quantize_i4 followed by the shared-input GEMM launch."""
+    k, ns = 4096, (4096, 1024, 1000)
+    print(f"case norm prologue m={m} grouped={grouped} add={with_add} weight={with_weight}", flush=True)
+    x = dev(syn.activations(m, k, seed=7 * m + grouped))
+    add = dev((np.random.default_rng(m).standard_normal((m, k)) * 0.5).astype(np.float16)) if with_add else None
+    nw = dev(np.random.default_rng(5).uniform(0.5, 1.5, k).astype(np.float16)) if with_weight else None
+    ws = [weights(n, k, k // 128 if grouped else 1, seed=n + m) for n in ns]
+    Bs, Ss = [dev(w) for w, _ in ws], [dev(s) for _, s in ws]
+    total, outs = ops.rmsnorm_rotate_quantize_gemm_i4_multi(x, add, nw, 1e-5, Bs, Ss)
+    if with_add:
+        want_total, q, s = ops.add_rmsnorm_rotate_and_quantize_i4(x, add, nw, 1e-5)
+        assert torch.equal(total, want_total) and torch.equal(total, x + add)
+    else:
+        assert total is None
+        q, s = ops.rmsnorm_rotate_and_quantize_i4(x, nw, 1e-5)
+    want = ops.gemm_i4_dequant_multi(q, Bs, s, Ss, 128)
+    for got, ref in zip(outs, want):
+        assert torch.equal(got.view(torch.int16), ref.view(torch.int16))
+
+
+def test_norm_prologue_argument_errors(ops):
+    x = torch.zeros(2, 4096, dtype=torch.float16, device="cuda")
+    B = torch.zeros(64, 2048, dtype=torch.uint8, device="cuda")
+    S = torch.ones(64, 1, dtype=torch.float16, device="cuda")
+    with pytest.raises(RuntimeError):
+        ops.rmsnorm_rotate_quantize_gemm_i4_multi(torch.zeros(5, 4096, dtype=torch.float16, device="cuda"), None, None, 1e-5, [B], [S])
+    with pytest.raises(RuntimeError):
+        ops.rmsnorm_rotate_quantize_gemm_i4_multi(x, x[:1], None, 1e-5, [B], [S])
+    with pytest.raises(RuntimeError):
+        ops.rmsnorm_rotate_quantize_gemm_i4_multi(x, None, torch.ones(100, dtype=torch.float16, device="cuda"), 1e-5, [B], [S])
