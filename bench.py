@@ -3,19 +3,20 @@
 
 A "step" is one pass over the seven linear layers of a Llama-2-7B decoder block at
 M = 2048 tokens (the configuration the headline metric is quoted on): per-token activation scales, per-channel
-weight scales, fp16 activations with 1 % outlier channels.  Per step:
+weight scales, fp16 activations with 1 % outlier channels.  Per step, issued the way a decoder layer issues it
+(--launches layer, the default):
 
-    rotate+quantise x[2048, 4096]          -> shared by q / k / v      (3 GEMMs 4096 x 4096)
-    rotate+quantise x[2048, 4096]          -> o_proj                   (1 GEMM  4096 x 4096)
-    rotate+quantise x[2048, 4096]          -> shared by gate / up      (2 GEMMs 11008 x 4096)
-    rotate+quantise x[2048, 11008] (172x64)-> down_proj                (1 GEMM  4096 x 11008)
+    rotate+quantise x[2048, 4096]          -> q, k, v as three weight matrices of ONE launch     (3 x 4096 x 4096)
+    rotate+quantise x[2048, 4096]          -> o_proj                                            (4096 x 4096)
+    rotate+quantise x[2048, 4096]          -> gate and up in ONE launch that stores silu(gate) * up   (2 x 11008 x 4096)
+    rotate+quantise x[2048, 11008] (172x64)-> down_proj                                         (4096 x 11008)
 
-`value` is integer tera-operations per second of the whole step (2*M*N*K summed over the
-seven GEMMs, divided by the wall time of the step including the four rotate+quantise
-launches), inputs resident in HBM.  The JSON line also carries the roofline of the
-dominant kernel (the GEMM, against the dense int8 MFMA peak), the roofline of the fused
-Hadamard-quant kernel (against HBM bandwidth), and the CPU oracle timed on a bounded
-sample of the same workload.
+--launches seven issues one GEMM launch per linear instead; whichever form is not the headline is timed and reported
+beside it.  `value` is integer tera-operations per second of the whole step (2*M*N*K summed over the seven
+contractions, divided by the wall time of the step including the four rotate+quantise launches), inputs resident in
+HBM.  The JSON line also carries the roofline of the dominant kernel (the GEMM, against the dense int8 MFMA peak), the
+roofline of the fused Hadamard-quant kernel (against HBM bandwidth), and the CPU oracle timed on a bounded sample of the
+same workload.
 
 Rotation modes (--hadamard): "fast" (default) runs the matrix-core kernels for all four launches: K = 4096 differs
 from the float32-butterfly codes in fewer than 1e-5 of the positions (measured live and reported; it is closer to the
@@ -23,7 +24,7 @@ reference's float64 transform than the float32 butterflies are), K = 11008 = 172
 order is defined by the reference for its dense factor).  "mixed" runs the bit-exact float32-butterfly kernel for
 K = 4096, "exact" for all four.  All modes are timed per kernel and reported either way.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline] [--hadamard fast]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline] [--hadamard fast] [--launches layer]
 """
 import argparse
 import json
