@@ -578,6 +578,19 @@ def main():
 
     us = wall_us(llama3_step_6bit, reps=args.steps)
     llama3["six_bit_matrix_instruction"] = {"us_per_layer": round(us, 1), "TOPS": round(ops3 / (us * 1e-6) / 1e12, 1)}
+
+    # ... with the quantisers writing the 6-bit format themselves (no encoding pass; float32 butterflies for K = 4096,
+    # matrix cores for K = 14336) and the projections that share an input in one launch: what a token-configuration layer
+    # with group-scaled weights issues for 256 rows or more
+    def llama3_step_6bit_direct():
+        for src, parts in groups3:
+            a6, ps = ops.rotate_and_quantize_f6(acts3[src])
+            out = ops.gemm_f6_dequant_multi(a6, [w3_6[n] for n in parts], ps, [w3[n][1] for n in parts])
+        return out
+
+    us = wall_us(llama3_step_6bit_direct, reps=args.steps)
+    llama3["six_bit_direct_format,shared_launches"] = {"us_per_layer": round(us, 1),
+                                                       "TOPS": round(ops3 / (us * 1e-6) / 1e12, 1)}
     # the same block at decode sizes (the linears of one layer of a Llama-3-8B decode step, batch x 1 token): graph
     # replays of 4 rotate-quantise + 4 GEMM launches (q/k/v and gate/up share their tokens), weights read once per step
     w3_bytes = int(sum(n * k // 2 + n * (k // 128) * 2 for _, n, k, _ in L3))

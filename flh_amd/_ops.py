@@ -672,6 +672,42 @@ def add_rmsnorm_rotate_and_quantize_i4(x, add, weight, eps, hadamard=True, clip_
     return total, q, s
 
 
+def rotate_and_quantize_f6(x, hadamard=True, clip_ratio=1.0, norm_weight=None, eps=None, add=None):
+    """rotate_and_quantize_i4 (one scale per token) with the codes written in the 6-bit operand format of gemm_f6_*
+    directly: x [M, K] fp16 -> (encoded [M, K / 128 * 96] u8, scales [M, 1] fp16), the bytes of encode_f6(q).
+    K = 512 .. 8192 a power of two (float32 butterflies, `hadamard` True / "exact" / False) -- optionally behind RMSNorm
+    (`eps` given; `norm_weight` [K] fp16 or None) and a residual addition (`add` [M, K]: the sum is returned first) --
+    or K = 11008 / 14336 on the matrix cores (`hadamard` True / "fast")."""
+    _check(x.is_cuda and x.dtype == torch.float16 and x.dim() == 2 and x.is_contiguous(),
+           "Input tensor must be a contiguous 2D float16 CUDA tensor")
+    M, K = x.shape
+    dense = K in (11008, 14336)
+    _check(dense or K in (512, 1024, 2048, 4096, 8192), "Last dimension must be a power of two in 512 .. 8192, 11008 or 14336")
+    if dense:
+        _check(hadamard in (True, "fast") and eps is None and add is None, "K = 11008 / 14336: matrix-core rotation, no prologue")
+        mode = FLH_HAD_MFMA
+    else:
+        _check(hadamard in (True, False, None, "exact"), "power-of-two K: hadamard True / 'exact' / False")
+        mode = FLH_HAD_F32 if hadamard in (True, "exact") else FLH_HAD_NONE
+    _check(add is None or eps is not None, "the residual addition comes with the RMSNorm prologue (eps)")
+    if add is not None:
+        _check(add.is_cuda and add.dtype == torch.float16 and add.shape == x.shape and add.is_contiguous()
+               and add.device == x.device, "add must be a contiguous float16 CUDA tensor of x's shape")
+    if norm_weight is not None:
+        _check(eps is not None and norm_weight.is_cuda and norm_weight.dtype == torch.float16 and norm_weight.is_contiguous()
+               and norm_weight.numel() == K and norm_weight.device == x.device,
+               "norm_weight must be a contiguous float16 CUDA tensor of K values (with eps)")
+    enc = torch.empty((M, K // 128 * 96), dtype=torch.uint8, device=x.device)
+    s = torch.empty((M, 1), dtype=torch.float16, device=x.device)
+    total = torch.empty_like(x) if add is not None else None
+    if M:
+        _run("flh_rotate_quant_f6", x.device, x.data_ptr(), add.data_ptr() if add is not None else None,
+             total.data_ptr() if total is not None else None, 1 if eps is not None else 0,
+             norm_weight.data_ptr() if norm_weight is not None else None, float(eps or 0.0), enc.data_ptr(), s.data_ptr(), M, K,
+             mode, float(clip_ratio), _stream(x))
+    return (total, enc, s) if add is not None else (enc, s)
+
+
 def rotate_and_quantize_i4(x, hadamard=True, had_group=0, scale_group=0, clip_ratio=1.0, return_rotated=False):
     """Whole-row online rotation + symmetric int4 quantise + pack: x [M, K] fp16 ->
     (q [M, K/2] u8, scales [M, 1 or K/scale_group] fp16 [, y [M, K] fp16]).

@@ -29,6 +29,7 @@
 
 #include "lane_ops.h"
 #include "quant_pack.h"
+#include "f6_codes.h"
 
 namespace flh {
 namespace {
@@ -302,7 +303,10 @@ __device__ __forceinline__ v2i quantise_half_block(const unsigned (&y)[8], float
 // x2 = up -- what the reference's MLP hands to the quantiser of down_proj (flh/quantized_model/modeling_llama.py:522-526).
 // Both rows are staged in LDS the same way and combined in place before the first tile is read, so the product never
 // goes to memory.
-template <int DT, bool SPLIT, bool SILU = false>
+//
+// F6 (long batches only): the codes leave in the operand format of the 6-bit matrix instruction (gemm_f6.hip) -- q is
+// then the encoded matrix of M rows, K-slab-major blocks of 96 bytes per 128 codes and row.
+template <int DT, bool SPLIT, bool SILU = false, bool F6 = false>
 __global__ __launch_bounds__(512) void rotate_quant_mfma_dense_kernel(const __half* __restrict__ x,
                                                                        uint8_t* __restrict__ q,
                                                                        __half* __restrict__ scales,
@@ -310,6 +314,7 @@ __global__ __launch_bounds__(512) void rotate_quant_mfma_dense_kernel(const __ha
                                                                        float inv_norm, float clip,
                                                                        const __half* __restrict__ x2 = nullptr) {
   static_assert(!SILU || SPLIT, "the SwiGLU prologue works on the row staged in LDS");
+  static_assert(!F6 || !SPLIT, "6-bit output is a prefill format");
   constexpr int D = DenseFactor<DT>::D, K = D * 64, NFRAG = 2 * DT * DT;
   extern __shared__ __align__(1024) h8 mfrag[];        // [kb][s][nt][lane], then the maxima
   float* red = (float*)(mfrag + NFRAG * 64);           // [parity][row slot][mt]
@@ -494,7 +499,21 @@ __global__ __launch_bounds__(512) void rotate_quant_mfma_dense_kernel(const __ha
 #pragma unroll
         for (int u = 0; u < 8; ++u) y[u] = scale_pack_f16(w[nt][2 * u], w[nt][2 * u + 1], c);
         const v2i out = quantise_half_block<decltype(careful_tag)::value>(y, rinv, hb);
-        if (32 * nt + 31 < D || 32 * nt + col < D) *(v2i*)(qr + (32 * nt + col) * 32) = out;
+        if constexpr (F6) {
+          // this lane: codes 32 mt + 16 h + 0 .. 15 of block j' = 32 nt + col, i.e. 12 bytes at byte 12 h of the piece
+          // (half mt, sub-block j' % 2) of 128-code block j' / 2
+          const int jp = 32 * nt + col;
+          const unsigned long long lo = bf6_of_nibbles((unsigned)out[0]), hi = bf6_of_nibbles((unsigned)out[1]);
+          unsigned* dst = (unsigned*)(q + ((size_t)(jp >> 1) * M + (valid ? row : M - 1)) * kF6BlockBytes + 48 * mt +
+                                      24 * (jp & 1) + 12 * h);
+          if (32 * nt + 31 < D || jp < D) {
+            dst[0] = (unsigned)lo;
+            dst[1] = (unsigned)(lo >> 32) | ((unsigned)hi << 16);
+            dst[2] = (unsigned)(hi >> 16);
+          }
+        } else {
+          if (32 * nt + 31 < D || 32 * nt + col < D) *(v2i*)(qr + (32 * nt + col) * 32) = out;
+        }
       }
     };
     if (careful) emit(std::true_type{});
@@ -553,22 +572,24 @@ int launch_dense_silu(const __half* gate, const __half* up, uint8_t* q, __half* 
 }
 
 template <int DT>
-int launch_dense(const __half* x, uint8_t* q, __half* scales, uint32_t M, float clip, hipStream_t stream) {
+int launch_dense(const __half* x, uint8_t* q, __half* scales, uint32_t M, float clip, hipStream_t stream, bool f6 = false) {
   constexpr int NFRAG = 2 * DT * DT;
   constexpr int K = DenseFactor<DT>::D * 64;
   const h8* table = nullptr;
   if (int rc = dense_table<DT>(&table)) return rc;
   // short batches take one row per workgroup (SPLIT: exactly one -- the grid is M -- with the row staged in LDS),
-  // long ones four
-  const bool split = M <= 256;
+  // long ones four; 6-bit output (a prefill format) always takes the long-batch kernel
+  const bool split = M <= 256 && !f6;
   const size_t smem = (size_t)NFRAG * 1024 + 64 + (split ? (size_t)DT * 4096 : 0);   // factor fragments, the pairs' maxima, the row
-  auto kern = split ? rotate_quant_mfma_dense_kernel<DT, true> : rotate_quant_mfma_dense_kernel<DT, false>;
+  auto kern = f6 ? rotate_quant_mfma_dense_kernel<DT, false, false, true>
+                 : split ? rotate_quant_mfma_dense_kernel<DT, true> : rotate_quant_mfma_dense_kernel<DT, false>;
   constexpr int kThreadsDense = 512;
-  static std::atomic<bool> attr[2] = {{false}, {false}};   // set-up is idempotent: a race only repeats it
-  if (!attr[split].load(std::memory_order_acquire)) {
+  static std::atomic<bool> attr[3] = {{false}, {false}, {false}};   // set-up is idempotent: a race only repeats it
+  const int variant = f6 ? 2 : split;
+  if (!attr[variant].load(std::memory_order_acquire)) {
     if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess)
       return fail(FLH_ELAUNCH, "rotate_quant: cannot reserve %zu bytes of LDS", smem);
-    attr[split].store(true, std::memory_order_release);
+    attr[variant].store(true, std::memory_order_release);
   }
   const unsigned blocks = split ? M : ((M + 3) / 4 < 256u ? (M + 3) / 4 : 256u);
   hipLaunchKernelGGL(kern, dim3(blocks), dim3(kThreadsDense), smem, stream, x, q, scales, table, M,
@@ -593,6 +614,14 @@ int launch_silu_mul_rotate_quant_mfma(const __half* gate, const __half* up, uint
   if (K == 11008) return launch_dense_silu<6>(gate, up, q, scales, M, stream);
   if (K == 14336) return launch_dense_silu<7>(gate, up, q, scales, M, stream);
   return fail(FLH_EINVAL, "silu_mul_rotate_quant: K = %u is not supported (11008 or 14336)", K);
+}
+
+// launcher used by flh_rotate_quant_f6 (fwht_quant.hip): the dense-factor sizes with 6-bit output
+int launch_rotate_quant_mfma_f6(const __half* x, uint8_t* encoded, __half* scales, uint32_t M, uint32_t K, float clip,
+                                hipStream_t stream) {
+  if (K == 11008) return launch_dense<6>(x, encoded, scales, M, clip, stream, true);
+  if (K == 14336) return launch_dense<7>(x, encoded, scales, M, clip, stream, true);
+  return fail(FLH_EINVAL, "rotate_quant_f6 (matrix-core mode): K = %u is not supported", K);
 }
 
 // launcher used by flh_rotate_quant_i4 (fwht_quant.hip)

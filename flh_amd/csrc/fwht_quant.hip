@@ -170,22 +170,8 @@ __device__ __forceinline__ void group_finish(const h2 (&v)[4], int lir, bool val
                  y45 = __builtin_bit_cast(unsigned, v[2]), y67 = __builtin_bit_cast(unsigned, v[3]);
   const unsigned w = careful ? nibbles8<true>(y01, y23, y45, y67, r, hb) : nibbles8<false>(y01, y23, y45, y67, r, hb);
   if constexpr (F6) {
-    const unsigned long long own = bf6_of_nibbles(w);
-    const unsigned lo = (unsigned)own, hi = (unsigned)(own >> 32);
-    constexpr int kDppQuadXor3 = 0x1B;                  // quad_perm:[3,2,1,0]
-    const int role = lir & 3;                           // position of this lane's 48 bits inside the 24-byte piece
-    // all four moves run in every lane (a cross-lane read inside a divergent branch would see disabled lanes)
-    const unsigned x1lo = (unsigned)dpp_i<kDppQuadXor1>((int)lo), x1hi = (unsigned)dpp_i<kDppQuadXor1>((int)hi);
-    const unsigned x3lo = (unsigned)dpp_i<kDppQuadXor3>((int)lo), x3hi = (unsigned)dpp_i<kDppQuadXor3>((int)hi);
-    const unsigned nlo = role == 1 ? x3lo : x1lo, nhi = role == 1 ? x3hi : x1hi;
-    const unsigned long long next = (unsigned long long)nlo | ((unsigned long long)nhi << 32);
-    const unsigned long long word = role == 0 ? own | (next << 48) : role == 1 ? (own >> 16) | (next << 32)
-                                                                              : (own >> 32) | (next << 16);
-    if (valid && role < 3) {
-      const size_t block = (size_t)(row % groups_per_token) * tokens + row / groups_per_token;
-      uint8_t* dst = q + block * kF6BlockBytes + 48 * ((lir >> 2) & 1) + 24 * (lir >> 3) + 8 * role;
-      *(v2i*)dst = v2i{(int)(unsigned)word, (int)(unsigned)(word >> 32)};
-    }
+    const size_t block = (size_t)(row % groups_per_token) * tokens + row / groups_per_token;
+    f6_store_chunk(w, lir, q + block * kF6BlockBytes, valid);
   }
   if (valid) {
     using offset_t = std::conditional_t<OFF32, uint32_t, size_t>;
@@ -334,14 +320,15 @@ __global__ __launch_bounds__(256) void rotate_quant_wave_kernel(const __half* __
                                                                 __half* __restrict__ y_out, uint32_t M, float norm,
                                                                 float clip, const __half* __restrict__ rms_weight = nullptr,
                                                                 float rms_eps = 0.f, const __half* add = nullptr,
-                                                                __half* sum_out = nullptr) {
+                                                                __half* sum_out = nullptr, uint32_t f6 = 0) {
   constexpr int K = 512 * J;
   const uint32_t row = blockIdx.x * 4u + (threadIdx.x >> 6);
   if (row >= M) return;  // wave-uniform
-  rotate_quant_row<J, HAD, EXACT_NORM, RMS>(x + (size_t)row * K, q + (size_t)row * (K / 2), scales + row,
+  // f6: q is the encoded matrix of M rows in the 6-bit operand format instead of [M, K / 2] nibbles
+  rotate_quant_row<J, HAD, EXACT_NORM, RMS>(x + (size_t)row * K, f6 ? q : q + (size_t)row * (K / 2), scales + row,
                                             y_out ? y_out + (size_t)row * K : nullptr, norm, clip, rms_weight, rms_eps,
                                             add ? add + (size_t)row * K : nullptr,
-                                            add ? sum_out + (size_t)row * K : nullptr);
+                                            add ? sum_out + (size_t)row * K : nullptr, f6 ? M : 0u, row);
 }
 
 constexpr int kGenericThreads = 1024;      // one workgroup per compute unit (LDS): two waves per SIMD hide latencies
@@ -559,7 +546,7 @@ bool factor_hadamard(uint32_t K, int* Kd, int* P) {
 
 template <int J>
 int launch_wave(const __half* x, uint8_t* q, __half* s, __half* y, uint32_t M, bool had, float clip,
-                hipStream_t stream) {
+                hipStream_t stream, uint32_t f6 = 0) {
   constexpr int K = 512 * J;
   int lg = 0;
   while ((1 << lg) < K) ++lg;
@@ -567,14 +554,14 @@ int launch_wave(const __half* x, uint8_t* q, __half* s, __half* y, uint32_t M, b
   const dim3 grid((M + 3) / 4), block(256);
   if (!had)
     hipLaunchKernelGGL((rotate_quant_wave_kernel<J, false, true>), grid, block, 0, stream, x, q, s, y, M, 1.0f, clip,
-                       (const __half*)nullptr, 0.f, (const __half*)nullptr, (__half*)nullptr);
+                       (const __half*)nullptr, 0.f, (const __half*)nullptr, (__half*)nullptr, f6);
   else if (even)
     hipLaunchKernelGGL((rotate_quant_wave_kernel<J, true, true>), grid, block, 0, stream, x, q, s, y, M,
                        1.0f / (float)(1 << (lg / 2)), clip, (const __half*)nullptr, 0.f, (const __half*)nullptr,
-                       (__half*)nullptr);
+                       (__half*)nullptr, f6);
   else
     hipLaunchKernelGGL((rotate_quant_wave_kernel<J, true, false>), grid, block, 0, stream, x, q, s, y, M,
-                       sqrtf((float)K), clip, (const __half*)nullptr, 0.f, (const __half*)nullptr, (__half*)nullptr);
+                       sqrtf((float)K), clip, (const __half*)nullptr, 0.f, (const __half*)nullptr, (__half*)nullptr, f6);
   return check_launch("rotate_quant_wave");
 }
 
@@ -620,20 +607,21 @@ constexpr uint32_t kRow8MaxRows = 512;
 
 template <int J>
 int launch_wave_rms(const __half* x, const __half* w, float eps, uint8_t* q, __half* s, __half* y, uint32_t M, bool had,
-                    float clip, hipStream_t stream, const __half* add = nullptr, __half* sum_out = nullptr) {
+                    float clip, hipStream_t stream, const __half* add = nullptr, __half* sum_out = nullptr,
+                    uint32_t f6 = 0) {
   constexpr int K = 512 * J;
   int lg = 0;
   while ((1 << lg) < K) ++lg;
   const dim3 grid((M + 3) / 4), block(256);
   if (!had)
     hipLaunchKernelGGL((rotate_quant_wave_kernel<J, false, true, true>), grid, block, 0, stream, x, q, s, y, M, 1.0f,
-                       clip, w, eps, add, sum_out);
+                       clip, w, eps, add, sum_out, f6);
   else if (lg % 2 == 0)
     hipLaunchKernelGGL((rotate_quant_wave_kernel<J, true, true, true>), grid, block, 0, stream, x, q, s, y, M,
-                       1.0f / (float)(1 << (lg / 2)), clip, w, eps, add, sum_out);
+                       1.0f / (float)(1 << (lg / 2)), clip, w, eps, add, sum_out, f6);
   else
     hipLaunchKernelGGL((rotate_quant_wave_kernel<J, true, false, true>), grid, block, 0, stream, x, q, s, y, M,
-                       sqrtf((float)K), clip, w, eps, add, sum_out);
+                       sqrtf((float)K), clip, w, eps, add, sum_out, f6);
   return check_launch("rmsnorm_rotate_quant_wave");
 }
 
@@ -696,6 +684,8 @@ int launch_rotate_quant_mfma(const __half* x, uint8_t* q, __half* scales, uint32
 bool rotate_quant_mfma_supports(uint32_t K);
 int launch_silu_mul_rotate_quant_mfma(const __half* gate, const __half* up, uint8_t* q, __half* scales, uint32_t M,
                                       uint32_t K, hipStream_t stream);
+int launch_rotate_quant_mfma_f6(const __half* x, uint8_t* encoded, __half* scales, uint32_t M, uint32_t K, float clip,
+                                hipStream_t stream);
 
 }  // namespace flh
 
@@ -806,6 +796,51 @@ extern "C" int flh_add_rmsnorm_rotate_quant_i4(const flh_half* x, const flh_half
     case 4: return launch_wave_rms<4>(xh, wh, eps, q_packed, sh, nullptr, M, had, clip_ratio, st, ah, oh);
     case 8: return launch_wave_rms<8>(xh, wh, eps, q_packed, sh, nullptr, M, had, clip_ratio, st, ah, oh);
     default: return launch_wave_rms<16>(xh, wh, eps, q_packed, sh, nullptr, M, had, clip_ratio, st, ah, oh);
+  }
+}
+
+extern "C" int flh_rotate_quant_f6(const flh_half* x, const flh_half* add, flh_half* sum_out, int rmsnorm,
+                                   const flh_half* weight, float eps, uint8_t* encoded, flh_half* scales, uint32_t M,
+                                   uint32_t K, int hadamard, float clip_ratio, void* stream) {
+  const char* who = "rotate_quant_f6";
+  if (!x || !encoded || !scales) return fail(FLH_EINVAL, "%s: null pointer", who);
+  if (misaligned16(x, encoded)) return fail(FLH_EINVAL, "%s: x and encoded must be 16-byte aligned", who);
+  if ((add == nullptr) != (sum_out == nullptr)) return fail(FLH_EINVAL, "%s: add and sum_out come together or not at all", who);
+  if (add && !rmsnorm) return fail(FLH_EINVAL, "%s: the residual addition comes with the RMSNorm prologue", who);
+  if (add && misaligned16(add, sum_out)) return fail(FLH_EINVAL, "%s: add and sum_out must be 16-byte aligned", who);
+  if (sum_out && ((const void*)sum_out == (const void*)x || (const void*)sum_out == (const void*)add))
+    return fail(FLH_EINVAL, "%s: sum_out must not be x or add", who);
+  if (weight && (!rmsnorm || misaligned16(weight))) return fail(FLH_EINVAL, "%s: weight needs rmsnorm != 0 and 16-byte alignment", who);
+  if (!(clip_ratio > 0.f)) return fail(FLH_EINVAL, "%s: clip_ratio must be positive", who);
+  if (!(eps >= 0.f)) return fail(FLH_EINVAL, "%s: eps must not be negative", who);
+  if (M == 0) return FLH_OK;
+  const __half *xh = (const __half*)x, *ah = (const __half*)add, *wh = (const __half*)weight;
+  __half *sh = (__half*)scales, *oh = (__half*)sum_out;
+  hipStream_t st = (hipStream_t)stream;
+  if (hadamard == FLH_HAD_MFMA) {
+    if (rmsnorm) return fail(FLH_EINVAL, "%s: the matrix-core rotation has no RMSNorm prologue", who);
+    if (K != 11008 && K != 14336) return fail(FLH_EINVAL, "%s: matrix-core rotation with 6-bit output: K (%u) must be 11008 or 14336", who, K);
+    return launch_rotate_quant_mfma_f6(xh, encoded, sh, M, K, clip_ratio, st);
+  }
+  if (hadamard != FLH_HAD_NONE && hadamard != FLH_HAD_F32) return fail(FLH_EINVAL, "%s: unknown hadamard mode %d", who, hadamard);
+  if (K % 512 || !is_pow2(K / 512) || K > 8192)
+    return fail(FLH_EINVAL, "%s: K (%u) must be 512, 1024, 2048, 4096 or 8192 (or 11008 / 14336 on the matrix cores)", who, K);
+  const bool had = hadamard != FLH_HAD_NONE;
+  if (rmsnorm) {
+    switch (K / 512) {
+      case 1: return launch_wave_rms<1>(xh, wh, eps, encoded, sh, nullptr, M, had, clip_ratio, st, ah, oh, 1);
+      case 2: return launch_wave_rms<2>(xh, wh, eps, encoded, sh, nullptr, M, had, clip_ratio, st, ah, oh, 1);
+      case 4: return launch_wave_rms<4>(xh, wh, eps, encoded, sh, nullptr, M, had, clip_ratio, st, ah, oh, 1);
+      case 8: return launch_wave_rms<8>(xh, wh, eps, encoded, sh, nullptr, M, had, clip_ratio, st, ah, oh, 1);
+      default: return launch_wave_rms<16>(xh, wh, eps, encoded, sh, nullptr, M, had, clip_ratio, st, ah, oh, 1);
+    }
+  }
+  switch (K / 512) {
+    case 1: return launch_wave<1>(xh, encoded, sh, nullptr, M, had, clip_ratio, st, 1);
+    case 2: return launch_wave<2>(xh, encoded, sh, nullptr, M, had, clip_ratio, st, 1);
+    case 4: return launch_wave<4>(xh, encoded, sh, nullptr, M, had, clip_ratio, st, 1);
+    case 8: return launch_wave<8>(xh, encoded, sh, nullptr, M, had, clip_ratio, st, 1);
+    default: return launch_wave<16>(xh, encoded, sh, nullptr, M, had, clip_ratio, st, 1);
   }
 }
 

@@ -5,6 +5,7 @@
 #pragma once
 #include "lane_ops.h"
 #include "quant_pack.h"
+#include "f6_codes.h"
 
 namespace flh {
 namespace {
@@ -90,11 +91,16 @@ __device__ __forceinline__ v4i add_h8(v4i a, v4i b) {
 // that sum is also stored to sum_row -- the residual stream of a decoder layer (modeling_llama.py:600-618:
 // hidden = residual + attention output; residual = hidden; hidden = norm(hidden)) without a launch of its own.
 // sum_row overlaps neither input.
+//
+// f6_rows > 0: the codes leave in the operand format of the 6-bit matrix instruction (gemm_f6.hip: K-slab-major blocks
+// of 96 bytes per 128 codes and row) -- q_row is then the BASE of the encoded matrix, f6_rows its row count and f6_row
+// this row's index.
 template <int J, bool HAD, bool EXACT_NORM, bool RMS = false>
 __device__ __forceinline__ void rotate_quant_row(const __half* __restrict__ x_row, uint8_t* q_row, __half* scale_dst,
                                                  __half* y_row, float norm, float clip,
                                                  const __half* __restrict__ rms_weight = nullptr, float rms_eps = 0.f,
-                                                 const __half* add_row = nullptr, __half* sum_row = nullptr) {
+                                                 const __half* add_row = nullptr, __half* sum_row = nullptr,
+                                                 uint32_t f6_rows = 0, uint32_t f6_row = 0) {
   constexpr int K = 512 * J, N = 8 * J;
   const int lane = threadIdx.x & 63;
   const int c = lane_chunk(lane);
@@ -234,9 +240,16 @@ __device__ __forceinline__ void rotate_quant_row(const __half* __restrict__ x_ro
   const h2 hb = {(_Float16)mx, (_Float16)mx};
   unsigned* qr = (unsigned*)q_row + c;
 #pragma unroll
-  for (int j = 0; j < J; ++j)
-    qr[j * 64] = careful ? nibbles8<true>(yp[4 * j], yp[4 * j + 1], yp[4 * j + 2], yp[4 * j + 3], r, hb)
-                         : nibbles8<false>(yp[4 * j], yp[4 * j + 1], yp[4 * j + 2], yp[4 * j + 3], r, hb);
+  for (int j = 0; j < J; ++j) {
+    const unsigned w = careful ? nibbles8<true>(yp[4 * j], yp[4 * j + 1], yp[4 * j + 2], yp[4 * j + 3], r, hb)
+                               : nibbles8<false>(yp[4 * j], yp[4 * j + 1], yp[4 * j + 2], yp[4 * j + 3], r, hb);
+    if (f6_rows) {                                     // wave-uniform; chunk c of segment j sits in 128-code block 4 j + c / 16
+      const size_t block = (size_t)(4 * j + (c >> 4)) * f6_rows + f6_row;
+      f6_store_chunk(w, c & 15, q_row + block * kF6BlockBytes, true);
+    } else {
+      qr[j * 64] = w;
+    }
+  }
   if (lane == 0) *scale_dst = __builtin_bit_cast(__half, s);
 }
 

@@ -54,6 +54,16 @@ class LinearFLH(torch.nn.Module):
             self._w6_key = key
         return self._w6
 
+    def wants_six_bit(self, n_rows):
+        """Whether a call with `n_rows` per-token-quantised rows takes the 6-bit matrix instruction (a producer can then
+        write the activations in that format directly, rotate_and_quantize_f6)."""
+        if self.six_bit is False or n_rows < self.six_bit_min_rows or self.in_features % 128 or not self.w_packed.is_cuda:
+            return False
+        cols = self.w_scale.view(self.out_features, -1).size(1)
+        if cols == 1:
+            return self.six_bit is True
+        return cols == self.in_features // 128 and self.weight_group_size == 128
+
     def _six_bit_applies(self, rows, a_scale, w_scale, group):
         if self.six_bit is False or not (rows.is_cuda and rows.size(0) >= self.six_bit_min_rows
                                          and self.in_features % 128 == 0):

@@ -196,9 +196,23 @@ class W4A4DecoderLayer(torch.nn.Module):
             self._norm16[name] = hit
         return hit[1]
 
-    def _token_quant(self, stage, x, norm=None, norm_name=None):
+    _F6_WIDTHS = (512, 1024, 2048, 4096, 8192, 11008, 14336)
+
+    def _six_bit_for(self, consumers, n_rows, width):
+        """Whether the quantiser in front of `consumers` should write the 6-bit operand format directly: every consumer
+        would re-encode the nibbles for the 6-bit matrix instruction anyway."""
+        return (bool(consumers) and self.activation == "token" and self.fused and self.record is None
+                and width in self._F6_WIDTHS and all(l.wants_six_bit(n_rows) for l in consumers))
+
+    def _token_quant(self, stage, x, norm=None, norm_name=None, consumers=()):
         """Whole-row rotation + one scale per token (after RMSNorm when `norm` is given)."""
         rows = x.reshape(-1, x.size(-1)).contiguous()
+        if self._six_bit_for(consumers, rows.size(0), rows.size(1)):
+            if norm is not None:
+                q, s = _ops().rotate_and_quantize_f6(rows, norm_weight=self._norm_weight16(norm_name, norm), eps=norm.eps)
+            else:
+                q, s = _ops().rotate_and_quantize_f6(rows)
+            return s.view(*x.shape[:-1], 1), None, q.view(*x.shape[:-1], -1)
         if norm is not None and self.fused:
             q, s = _ops().rmsnorm_rotate_and_quantize_i4(rows, self._norm_weight16(norm_name, norm), norm.eps)
         else:
@@ -208,9 +222,9 @@ class W4A4DecoderLayer(torch.nn.Module):
         self._tap(stage + ".scales", s)
         return s.view(*x.shape[:-1], 1), None, q.view(*x.shape[:-1], -1)
 
-    def _norm_quant(self, stage, norm, norm_name, quantizer, x):
+    def _norm_quant(self, stage, norm, norm_name, quantizer, x, consumers=()):
         if self.activation == "token":
-            return self._token_quant(stage, x, norm, norm_name)
+            return self._token_quant(stage, x, norm, norm_name, consumers)
         if self.fused:
             q, s = _ops().rmsnorm_and_quantize_i4_gs(x.reshape(-1, x.size(-1)).contiguous(),
                                                      self._norm_weight16(norm_name, norm), norm.eps,
@@ -223,19 +237,24 @@ class W4A4DecoderLayer(torch.nn.Module):
         self._tap(stage + ".scales", s.reshape(-1, s.size(-1)))
         return s, z, q
 
-    def _residual_norm_quant(self, stage, norm, norm_name, quantizer, x, add):
+    def _residual_norm_quant(self, stage, norm, norm_name, quantizer, x, add, consumers=()):
         """(x + add, scales, zeros, codes): the residual addition (when `add` is given), the norm and the quantiser of
-        the linears that follow -- one launch where the whole-row path allows it, else the separate steps."""
+        the linears that follow (`consumers`) -- one launch where the whole-row path allows it, else the separate steps."""
         if add is None:
-            return (x,) + tuple(self._norm_quant(stage, norm, norm_name, quantizer, x))
+            return (x,) + tuple(self._norm_quant(stage, norm, norm_name, quantizer, x, consumers))
         k = x.size(-1)
+        if k in (512, 1024, 2048, 4096, 8192) and self._six_bit_for(consumers, x.numel() // k, k):
+            total, q, s = _ops().rotate_and_quantize_f6(
+                x.reshape(-1, k).contiguous(), norm_weight=self._norm_weight16(norm_name, norm), eps=norm.eps,
+                add=add.reshape(-1, k).contiguous())
+            return total.view(x.shape), s.view(*x.shape[:-1], 1), None, q.view(*x.shape[:-1], -1)
         if self.activation == "token" and self.fused and self.record is None and k in (512, 1024, 2048, 4096, 8192):
             total, q, s = _ops().add_rmsnorm_rotate_and_quantize_i4(
                 x.reshape(-1, k).contiguous(), add.reshape(-1, k).contiguous(), self._norm_weight16(norm_name, norm),
                 norm.eps)
             return total.view(x.shape), s.view(*x.shape[:-1], 1), None, q.view(*x.shape[:-1], -1)
         x = x + add
-        return (x,) + tuple(self._norm_quant(stage, norm, norm_name, quantizer, x))
+        return (x,) + tuple(self._norm_quant(stage, norm, norm_name, quantizer, x, consumers))
 
     def _project(self, layers, q, s, z):
         if self.fused:
@@ -266,7 +285,7 @@ class W4A4DecoderLayer(torch.nn.Module):
                 x = total.view(x.shape)
         else:
             x, s, z, q = self._residual_norm_quant("attn_in", self.input_layernorm, "input_layernorm",
-                                                   self.attn_quantizer1, x, add)
+                                                   self.attn_quantizer1, x, add, (self.q_proj, self.k_proj, self.v_proj))
             qs, ks, vs = self._project([self.q_proj, self.k_proj, self.v_proj], q, s, z)
         self._tap("q_proj", qs), self._tap("k_proj", ks), self._tap("v_proj", vs)
         static = isinstance(kv_cache, StaticKVCache._Layer)
@@ -332,7 +351,8 @@ class W4A4DecoderLayer(torch.nn.Module):
                 and self.hidden_size == 4096):
             # decode: the quantiser runs inside the GEMM's own launch (same bits as the two launches)
             return x, self.o_proj.forward_online(out, hadamard="exact"), cache
-        s, z, q = self._token_quant("attn_out", out) if self.activation == "token" else self._group_quant("attn_out", self.attn_quantizer2, out)
+        s, z, q = (self._token_quant("attn_out", out, consumers=(self.o_proj,)) if self.activation == "token"
+                   else self._group_quant("attn_out", self.attn_quantizer2, out))
         y = self.o_proj(q, s, z, x_is_packed=True)
         self._tap("o_proj", y)
         return x, y, cache
@@ -351,14 +371,10 @@ class W4A4DecoderLayer(torch.nn.Module):
         cols = g.w_scale.view(g.out_features, -1).size(1)
         return g.bias is None and self.up_proj.bias is None and (cols == 1 or (g.weight_group_size == 128 and cols == g.in_features // 128))
 
-    def _six_bit_gate_up(self, q, s):
-        """Whether gate / up would take the 6-bit matrix instruction for these activations (faster than the int8 launch
-        that fuses the SwiGLU product when the weights carry group scales)."""
-        rows = q.reshape(-1, q.size(-1))
-        g = self.gate_proj
-        group = g.weight_group_size if g.weight_group_size > 0 else (g.in_group_size or 128)
-        return all(l._six_bit_applies(rows, s.reshape(rows.size(0), -1), l.w_scale.view(l.out_features, -1), group)
-                   for l in (self.gate_proj, self.up_proj))
+    def _six_bit_gate_up(self, n_rows):
+        """Whether gate / up take the 6-bit matrix instruction for this many rows (faster than the int8 launch that fuses
+        the SwiGLU product when the weights carry group scales)."""
+        return all(l.wants_six_bit(n_rows) for l in (self.gate_proj, self.up_proj))
 
     def _group_quant(self, stage, quantizer, x):
         s, z, q = quantizer(x)
@@ -373,12 +389,13 @@ class W4A4DecoderLayer(torch.nn.Module):
     def _mlp(self, x, add):
         """mlp() on the residual stream x + add (add may be None); returns (that sum, the MLP's output)."""
         x, s, z, q = self._residual_norm_quant("mlp_in", self.post_attention_layernorm, "post_attention_layernorm",
-                                               self.mlp_quantizer1, x, add)
+                                               self.mlp_quantizer1, x, add, (self.gate_proj, self.up_proj))
         rows = q.numel() // q.size(-1)
         if (self.activation == "token" and self.fused and self.record is None and rows > 64
-                and self._swiglu_gemm_applies() and not self._six_bit_gate_up(q, s)):
+                and self._swiglu_gemm_applies() and not self._six_bit_gate_up(rows)):
             # prefill: gate and up in one launch that stores silu(gate) * up only (no fp16 [M, I] round trips)
-            s, z, q = self._token_quant("mlp_mid", LinearFLH.forward_swiglu(self.gate_proj, self.up_proj, q, s))
+            s, z, q = self._token_quant("mlp_mid", LinearFLH.forward_swiglu(self.gate_proj, self.up_proj, q, s),
+                                        consumers=(self.down_proj,))
             return x, self.down_proj(q, s, z, x_is_packed=True)
         gate, up = self._project([self.gate_proj, self.up_proj], q, s, z)
         self._tap("gate_proj", gate), self._tap("up_proj", up)
@@ -390,7 +407,7 @@ class W4A4DecoderLayer(torch.nn.Module):
         elif self.activation == "token":
             # (the library's product kernel when fused, so that every fused path sees the same fp16 product)
             mid = _ops().silu_mul(gate, up) if self.fused else torch.nn.functional.silu(gate) * up
-            s, z, q = self._token_quant("mlp_mid", mid)
+            s, z, q = self._token_quant("mlp_mid", mid, consumers=(self.down_proj,))
         elif self.fused and self.record is None:
             s, z, q = self._silu_mul_quant(gate, up)
         else:

@@ -172,6 +172,16 @@ int flh_gemm_f6_i32(const uint8_t* A6, const uint8_t* B6, int32_t* C, size_t M, 
  * (x [M, K] fp16 -> encoded [M, K/128 * 96], scales [M, K/128]); same codes and scales, no separate encoding pass. */
 int flh_group_quant_f6(const flh_half* x, uint8_t* encoded, flh_half* scales, uint32_t M, uint32_t K, int hadamard,
                        float scale_mul, void* stream);
+
+/* The whole-row rotation + per-token quantiser writing the 6-bit operand format directly (no flh_encode_f6 pass):
+ * encoded [M rows, K / 128 * 96 bytes] as flh_encode_f6 lays it out, scales [M].  hadamard FLH_HAD_NONE / FLH_HAD_F32 with
+ * K = 512 .. 8192 a power of two, optionally with the prologues of flh_rmsnorm_rotate_quant_i4 (rmsnorm != 0; weight [K]
+ * or null, eps) and flh_add_rmsnorm_rotate_quant_i4 (add / sum_out [M, K], both or neither, only with rmsnorm);
+ * FLH_HAD_MFMA with K = 11008 / 14336 (no prologue).  The bytes equal flh_encode_f6 of the nibble output of the
+ * corresponding flh_*rotate_quant_i4 call, the scales are the same.  No counterpart in the reference. */
+int flh_rotate_quant_f6(const flh_half* x, const flh_half* add, flh_half* sum_out, int rmsnorm, const flh_half* weight,
+                        float eps, uint8_t* encoded, flh_half* scales, uint32_t M, uint32_t K, int hadamard, float clip_ratio,
+                        void* stream);
 /* Group scales of 128 codes on the same instruction: b_scale [N, K/128], a_scale [M, K/128] (a_cols = K/128) or
  * [M] (a_cols = 1: one scale per token, applied after the groups).  The float32 accumulator makes the fold per
  * group one FMA per output; same bits as flh_gemm_i4_o16 with group = 128 on the same codes and scales. */

@@ -118,3 +118,25 @@ def test_six_bit_layer_gives_the_same_bits():
     assert six.q_proj._w6 is not None and six.down_proj._w6 is not None     # the 6-bit path really ran
     assert plain.q_proj._w6 is None and plain.down_proj._w6 is None
     assert torch.equal(a, b) and torch.equal(ka, kb) and torch.equal(va, vb)
+
+
+@pytest.mark.parametrize("six", [None, True])
+def test_token_layer_on_the_six_bit_path_gives_the_same_bits(six):
+    """Token configuration with group-scaled weights (the Llama-3 arrangement): from 256 rows on the layer's quantisers
+    write the 6-bit operand format directly and the linears run on the 6-bit matrix instruction (`six_bit=None`: by
+    default for group-scaled weights); outputs and cached keys / values must equal the int8 path's bit for bit."""
+    w, _ = make(seed=21)
+    group = 128 if six is None else 0                 # per-channel scales take the 6-bit path only when asked to
+    plain = W4A4DecoderLayer.from_float(w, 4, 2, activation="token", weight_group_size=group, six_bit=False)
+    fast = W4A4DecoderLayer.from_float(w, 4, 2, activation="token", weight_group_size=group, six_bit=six)
+    x = torch.randn(2, 150, 512, generator=torch.Generator().manual_seed(22)).half().cuda()
+    cos, sin = rotary_tables(torch.arange(150, device="cuda"), 128)
+    a, (ka, va) = plain(x, cos, sin)
+    b, (kb, vb) = fast(x, cos, sin)
+    assert fast.q_proj._w6 is not None and fast.o_proj._w6 is not None and fast.down_proj._w6 is not None
+    assert plain.q_proj._w6 is None
+    assert torch.equal(ka, kb) and torch.equal(va, vb)
+    assert torch.equal(a, b)
+    short = x[:, :8].contiguous()                     # 16 rows: below the threshold, the int8 / decode kernels
+    cs, ss = rotary_tables(torch.arange(8, device="cuda"), 128)
+    assert torch.equal(plain(short, cs, ss)[0], fast(short, cs, ss)[0])
