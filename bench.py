@@ -38,8 +38,8 @@ PEAK_INT8_TOPS = 5033.0   # 256 CU x 8192 int8 op/clk/CU x 2.4 GHz (dense)
 PEAK_HBM_GBS = 8000.0
 # measured HBM traffic per launch at M = 2048 (fetch + write), from the counter runs summarised in
 # profiles/llama7b_block_M2048_hbm_traffic.txt
-GEMM_TRAFFIC_BYTES = {"seven": int(((4 * 40.2 + 2 * 80.3 + 88.2) / 7 + (5 * 16.0 + 2 * 43.0) / 7) * 2 ** 20),
-                      "layer": None}
+GEMM_TRAFFIC_BYTES = {"seven": int(((4 * 40.2 + 2 * 80.2 + 88.2) / 7 + (5 * 16.0 + 2 * 43.0) / 7) * 2 ** 20),
+                      "layer": int(((83.5 + 40.2 + 147.0 + 88.2) / 4 + (48.0 + 16.0 + 43.0 + 16.0) / 4) * 2 ** 20)}
 QUANT4096_TRAFFIC_BYTES = int((16.2 + 4.02) * 2 ** 20)
 
 # (name, N, K, activation source) -- activation sources are quantised once and shared
