@@ -8,7 +8,9 @@ embedding, RoPE, attention, norms outside the fused launches and the head are st
 Weights are random (there are no checkpoints here): `random_init` draws fp16 weights layer by layer on the device and
 quantises them through the same kernels a loader would use.
 """
+import json
 import math
+import os
 
 import torch
 
@@ -34,6 +36,23 @@ class LlamaShape:
     @classmethod
     def llama2_7b(cls, num_layers=32):
         return cls(4096, 32, 32, 11008, num_layers, 32000, 1e-5, 10000.0)
+
+
+_ATTENTION = ("q_proj", "k_proj", "v_proj", "o_proj")
+_MLP = ("gate_proj", "up_proj", "down_proj")
+
+
+def reference_key(key):
+    """This model's state-dict key -> the key of the reference's model (a transformers LlamaForCausalLM subclass:
+    `model.layers.N.self_attn.q_proj.w_packed`, `model.layers.N.mlp.up_proj.w_scale`, `model.norm.weight`, `lm_head.weight`)."""
+    if key.startswith("lm_head."):
+        return key
+    parts = key.split(".")
+    if parts[0] == "layers" and parts[2] in _ATTENTION:
+        parts.insert(2, "self_attn")
+    elif parts[0] == "layers" and parts[2] in _MLP:
+        parts.insert(2, "mlp")
+    return "model." + ".".join(parts)
 
 
 class W4A4LlamaModel(torch.nn.Module):
@@ -77,6 +96,115 @@ class W4A4LlamaModel(torch.nn.Module):
                                                           activation))
                 del w
             model.layers = torch.nn.ModuleList(layers)
+        return model
+
+    # ------------------------------------------------------------------ the reference's checkpoint directory
+    def reference_state_dict(self):
+        """The state dict under the reference model's key names, float32 tensors as float16 (as its save_quantized
+        stores them, flh/quantized_model/modeling_llama.py:1099-1107)."""
+        out = {}
+        for key, value in self.state_dict().items():
+            value = value.detach().cpu()
+            out[reference_key(key)] = value.half() if value.dtype == torch.float32 else value
+        return out
+
+    def load_reference_state_dict(self, state, strict=True):
+        """Load a state dict with the reference model's key names (what its save_quantized wrote).  Keys this model has no
+        counterpart for (rotary buffers, quantiser settings) are ignored; with `strict`, every tensor of this model must
+        be present with its shape."""
+        own = self.state_dict()
+        missing = []
+        with torch.no_grad():
+            for key, dst in own.items():
+                src = state.get(reference_key(key))
+                if src is None:
+                    missing.append(reference_key(key))
+                    continue
+                if tuple(src.shape) != tuple(dst.shape):
+                    if src.numel() == dst.numel() and key.endswith("w_packed"):   # LinearFLHGS keeps [N, K/2], LinearFLH flat
+                        src = src.reshape(dst.shape)
+                    else:
+                        raise ValueError(f"{reference_key(key)}: shape {tuple(src.shape)}, expected {tuple(dst.shape)}")
+                dst.copy_(src.to(dst.dtype))
+        if strict and missing:
+            raise KeyError(f"missing in the checkpoint: {missing[:5]}{' ...' if len(missing) > 5 else ''}")
+        return missing
+
+    def save_quantized(self, save_directory, **quant_config):
+        """Write the reference's checkpoint directory (modeling_llama.py:1079-1137): `model.pt` (pickle protocol 4, the
+        reference model's key names), `quantization_config.json`, and `config.json` with the transformers fields that
+        define the architecture."""
+        from ..nn.checkpoint import QUANT_CONFIG_DEFAULTS
+        unknown = set(quant_config) - set(QUANT_CONFIG_DEFAULTS)
+        if unknown:
+            raise ValueError(f"unknown quantisation settings: {sorted(unknown)}")
+        os.makedirs(save_directory, exist_ok=True)
+        torch.save(self.reference_state_dict(), os.path.join(save_directory, "model.pt"), pickle_protocol=4)
+        first = self.layers[0].q_proj
+        grouped = first.w_scale.view(first.out_features, -1).size(1) > 1       # else one scale per output channel
+        settings = {**QUANT_CONFIG_DEFAULTS, "weight_group_size": first.weight_group_size if grouped else -1, **quant_config}
+        with open(os.path.join(save_directory, "quantization_config.json"), "w") as f:
+            json.dump(settings, f, indent=2)
+        sh = self.shape
+        with open(os.path.join(save_directory, "config.json"), "w") as f:
+            json.dump({"architectures": ["LlamaForCausalLM"], "model_type": "llama", "hidden_size": sh.hidden_size,
+                       "num_attention_heads": sh.num_heads, "num_key_value_heads": sh.num_kv_heads,
+                       "intermediate_size": sh.intermediate_size, "num_hidden_layers": sh.num_layers,
+                       "vocab_size": sh.vocab_size, "rms_norm_eps": sh.eps, "rope_theta": sh.rope_theta,
+                       "hidden_act": "silu", "torch_dtype": "float16",
+                       "flh_activation": self.activation}, f, indent=2)
+
+    @classmethod
+    def from_quantized(cls, load_directory, device="cuda", activation=None, fused=True):
+        """Build the model a checkpoint directory describes and load its tensors (modeling_llama.py:1139-1260).  The file
+        is read without executing anything from it (flh_amd.nn.checkpoint.read_state_dict).  `activation`: "group" (the
+        reference's own models) or "token"; default: what the directory's config says, else "group"."""
+        from ..nn.checkpoint import read_state_dict
+        with open(os.path.join(load_directory, "config.json")) as f:
+            cfg = json.load(f)
+        with open(os.path.join(load_directory, "quantization_config.json")) as f:
+            quant = json.load(f)
+        for key, want in (("weight_bits", 4), ("act_bits", 4)):
+            if quant.get(key, want) != want:
+                raise ValueError(f"{key} = {quant[key]}: this path is W4A4")
+        if not quant.get("weight_sym", True) or not quant.get("act_sym", True):
+            raise ValueError("asymmetric quantisation has no kernel on this path")
+        shape = LlamaShape(cfg["hidden_size"], cfg["num_attention_heads"],
+                           cfg.get("num_key_value_heads", cfg["num_attention_heads"]), cfg["intermediate_size"],
+                           cfg["num_hidden_layers"], cfg["vocab_size"], cfg.get("rms_norm_eps", 1e-5),
+                           cfg.get("rope_theta", 10000.0))
+        activation = activation or cfg.get("flh_activation", "group")
+        model = cls(shape, activation, quant.get("weight_group_size", 128), fused, device="cpu")
+        model.load_reference_state_dict(read_state_dict(os.path.join(load_directory, "model.pt")))
+        return model.to(device)
+
+    @classmethod
+    def from_float(cls, state, shape, activation="token", weight_group_size=128, fused=True, device="cuda"):
+        """Quantise a float Llama checkpoint given as a state dict with the transformers key names
+        (`model.layers.N.self_attn.q_proj.weight`, ..., `model.embed_tokens.weight`, `model.norm.weight`, `lm_head.weight`):
+        round-to-nearest through the same kernels a loader of quantised weights uses, one layer on the device at a time
+        (what the reference's `quantize` does layer by layer, modeling_llama.py:789-868, without its GPTQ option -- that is
+        flh_amd.nn.FLHGPTQ on a layer's float weights before this call)."""
+        model = cls(shape, activation, weight_group_size, fused, device="meta")
+        emb = state["model.embed_tokens.weight"]
+        model.embed_tokens = torch.nn.Embedding(shape.vocab_size, shape.hidden_size, device=device, dtype=torch.float16)
+        model.lm_head = torch.nn.Linear(shape.hidden_size, shape.vocab_size, bias=False, device=device, dtype=torch.float16)
+        model.norm = RMSNorm(shape.hidden_size, shape.eps).to(device)
+        layers = []
+        with torch.no_grad():
+            model.embed_tokens.weight.copy_(emb)
+            model.lm_head.weight.copy_(state.get("lm_head.weight", emb))       # tied embeddings: no separate head
+            model.norm.weight.copy_(state["model.norm.weight"].float())
+            for i in range(shape.num_layers):
+                pre = f"model.layers.{i}."
+                w = {name: state[pre + ("self_attn." if name in _ATTENTION else "mlp.") + name + ".weight"].to(device).half()
+                     for name in _ATTENTION + _MLP}
+                for name in ("input_layernorm", "post_attention_layernorm"):
+                    w[name] = state[pre + name + ".weight"].to(device).half()
+                layers.append(W4A4DecoderLayer.from_float(w, shape.num_heads, shape.num_kv_heads, shape.eps, 128,
+                                                          weight_group_size, fused, activation))
+                del w
+        model.layers = torch.nn.ModuleList(layers)
         return model
 
     def new_cache(self, batch, max_len):

@@ -314,3 +314,44 @@ def test_llama2_layer_8x512_against_the_oracle():
     err = np.linalg.norm(free.astype(np.float64) - got) / np.linalg.norm(got - host(x[:1]).astype(np.float64))
     print(f"  free-running oracle layer vs device (sequence 0): relative difference of the update {err:.3e}", flush=True)
     assert err < 0.3          # see the note on quantiser amplification in the decode-step test
+
+
+@pytest.mark.parametrize("activation,group", [("token", 128), ("token", 0), ("group", 128)])
+def test_float_checkpoint_to_quantised_directory_and_back(tmp_path, activation, group):
+    """A float checkpoint under the transformers key names -> W4A4LlamaModel.from_float -> save_quantized (the reference's
+    directory layout) -> from_quantized: the reloaded model gives the same logits bit for bit, for prefill and for a
+    decode step from the static cache."""
+    import math
+    shape = LlamaShape(512, 4, 2, 1024, 2, 320, 1e-5, 10000.0)
+    gen = torch.Generator().manual_seed(7)
+    state = {"model.embed_tokens.weight": torch.randn(shape.vocab_size, shape.hidden_size, generator=gen).half(),
+             "model.norm.weight": (torch.rand(shape.hidden_size, generator=gen) + 0.5).half(),
+             "lm_head.weight": (torch.randn(shape.vocab_size, shape.hidden_size, generator=gen) / math.sqrt(shape.hidden_size)).half()}
+    kv = shape.num_kv_heads * shape.head_dim
+    dims = {"self_attn.q_proj": (512, 512), "self_attn.k_proj": (kv, 512), "self_attn.v_proj": (kv, 512),
+            "self_attn.o_proj": (512, 512), "mlp.gate_proj": (1024, 512), "mlp.up_proj": (1024, 512), "mlp.down_proj": (512, 1024)}
+    for i in range(shape.num_layers):
+        for name, (n, k) in dims.items():
+            state[f"model.layers.{i}.{name}.weight"] = (torch.randn(n, k, generator=gen) / math.sqrt(k)).half()
+        for name in ("input_layernorm", "post_attention_layernorm"):
+            state[f"model.layers.{i}.{name}.weight"] = (torch.rand(shape.hidden_size, generator=gen) + 0.5).half()
+    print(f"case checkpoint round trip activation={activation} group={group}", flush=True)
+    with torch.no_grad():
+        model = W4A4LlamaModel.from_float(state, shape, activation=activation, weight_group_size=group)
+        model.save_quantized(tmp_path)
+        again = W4A4LlamaModel.from_quantized(tmp_path, device="cuda")
+        assert again.activation == activation
+        ids = torch.randint(0, shape.vocab_size, (2, 40), device="cuda", generator=torch.Generator(device="cuda").manual_seed(1))
+        pos = torch.arange(40, device="cuda")
+        want, got = model(ids, pos), again(ids, pos)
+        assert torch.isfinite(want).all() and torch.equal(want, got)
+        # a decode step from a static cache filled by the prefill
+        for m, ref in ((model, None), (again, None)):
+            cache = m.new_cache(2, 64)
+            cache.kv_len = 40
+            m(ids, pos, cache)
+            cache.kv_len = 41
+            step = m(ids[:, :1], torch.tensor([40], device="cuda"), cache)
+            if m is model:
+                first = step
+        assert torch.equal(first, step)

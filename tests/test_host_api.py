@@ -306,3 +306,43 @@ def test_torch_extension_loads_and_checks_tensors_without_a_device():
         ext.gemm_i4_dequant_o16(a, a, s, s)
     with pytest.raises(RuntimeError, match="CUDA"):
         ext.quant_and_pack_i4(torch.zeros(2, 128, dtype=torch.float16))
+
+
+def test_model_checkpoint_directory_uses_the_references_key_names(tmp_path):
+    """W4A4LlamaModel.save_quantized / from_quantized: the reference's directory layout (model.pt written with pickle
+    protocol 4 under the key names of its transformers model, quantization_config.json, config.json), read back without
+    executing anything from the file; every tensor survives the round trip."""
+    import json
+    import torch
+    from flh_amd.nn.checkpoint import read_state_dict
+    from flh_amd.quantized_model.llama import LlamaShape, W4A4LlamaModel, reference_key
+    assert reference_key("layers.3.q_proj.w_packed") == "model.layers.3.self_attn.q_proj.w_packed"
+    assert reference_key("layers.0.down_proj.w_scale") == "model.layers.0.mlp.down_proj.w_scale"
+    assert reference_key("layers.1.input_layernorm.weight") == "model.layers.1.input_layernorm.weight"
+    assert reference_key("norm.weight") == "model.norm.weight" and reference_key("lm_head.weight") == "lm_head.weight"
+    assert reference_key("embed_tokens.weight") == "model.embed_tokens.weight"
+    shape = LlamaShape(256, 4, 2, 512, 2, 100, 1e-6, 12345.0)
+    gen = torch.Generator().manual_seed(0)
+    model = W4A4LlamaModel(shape, activation="group", device="cpu")
+    with torch.no_grad():
+        for t in model.state_dict().values():
+            if t.dtype == torch.uint8:
+                t.copy_(torch.randint(0, 256, t.shape, dtype=torch.uint8, generator=gen))
+            else:
+                t.copy_(torch.randn(t.shape, generator=gen).half().to(t.dtype))
+    model.save_quantized(tmp_path, clip_ratio=0.9)
+    raw = read_state_dict(tmp_path / "model.pt")
+    assert "model.layers.1.mlp.gate_proj.w_packed" in raw and "model.norm.weight" in raw
+    assert raw["model.norm.weight"].dtype == torch.float16                      # float32 tensors are stored as float16
+    assert json.load(open(tmp_path / "quantization_config.json"))["clip_ratio"] == 0.9
+    cfg = json.load(open(tmp_path / "config.json"))
+    assert cfg["num_key_value_heads"] == 2 and cfg["rope_theta"] == 12345.0
+    again = W4A4LlamaModel.from_quantized(tmp_path, device="cpu")
+    assert again.shape.num_kv_heads == 2 and again.shape.eps == 1e-6 and again.activation == "group"
+    a, b = model.state_dict(), again.state_dict()
+    assert set(a) == set(b) and all(torch.equal(a[k], b[k]) for k in a)
+    # a checkpoint that lacks a tensor is refused
+    del raw["model.layers.0.self_attn.k_proj.w_scale"]
+    import pytest
+    with pytest.raises(KeyError):
+        W4A4LlamaModel(shape, activation="group", device="cpu").load_reference_state_dict(raw)
