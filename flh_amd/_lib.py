@@ -23,6 +23,8 @@ _SIG = {
                                    _c.c_int, _c.c_int, _c.c_int, _PTR]),
     "flh_gemm_i4_swiglu_o16": (_c.c_int, [_PTR, _PTR, _PTR, _PTR, _PTR, _PTR, _PTR, _c.c_size_t, _c.c_size_t, _c.c_size_t,
                                           _c.c_int, _c.c_int, _c.c_int, _PTR]),
+    "flh_gemm_f6_swiglu_o16": (_c.c_int, [_PTR, _PTR, _PTR, _PTR, _PTR, _PTR, _PTR, _c.c_size_t, _c.c_size_t, _c.c_size_t,
+                                          _c.c_int, _c.c_int, _PTR]),
     "flh_gemm_i4_o16_multi": (_c.c_int, [_PTR, _PTR, _c.c_int, _PTR, _PTR, _PTR, _PTR, _c.c_size_t, _c.c_size_t,
                                          _c.c_int, _c.c_int, _c.c_int, _PTR]),
     "flh_rotate_quant_gemm_i4_o16_multi": (_c.c_int, [_PTR, _c.c_int, _PTR, _PTR, _PTR, _PTR, _c.c_size_t, _c.c_size_t,

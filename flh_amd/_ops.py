@@ -338,6 +338,28 @@ def gemm_f6_dequant_o16_gs(A6, B6, A_scale, B_scale):
     return D
 
 
+def gemm_f6_swiglu(A6, B6_gate, B6_up, A_scale, gate_scale, up_scale):
+    """gemm_i4_swiglu on operands encoded by encode_f6 (or written by rotate_and_quantize_f6): fp16(fp16(silu(gate)) * up)
+    in one launch, gate / up = gemm_f6_dequant_o16[_gs](A6, B6_gate / B6_up, ...); scales all one column, or weight scales
+    [N, K/128] with A_scale [M, 1] or [M, K/128].  Same bits as gemm_i4_swiglu."""
+    M, N, K = _check_f6(A6, B6_gate)
+    _check(_check_f6(A6, B6_up) == (M, N, K), "gate and up must have the same shapes")
+    ng = K // 128
+    for t_ in (A_scale, gate_scale, up_scale):
+        _check(t_.is_cuda and t_.dtype == torch.float16 and t_.is_contiguous() and t_.dim() == 2 and t_.device == A6.device,
+               "scales must be contiguous 2D float16 CUDA tensors on the operands' device")
+    _check(up_scale.shape == gate_scale.shape and gate_scale.size(0) == N and gate_scale.size(1) in (1, ng),
+           "weight scales must be [N, 1] or [N, K/128], the same for gate and up")
+    _check(A_scale.size(0) == M and A_scale.size(1) in (1, ng) and (A_scale.size(1) == 1 or gate_scale.size(1) == ng),
+           "A_scale must be [M, 1], or [M, K/128] with group-scaled weights")
+    D = torch.empty((M, N), dtype=torch.float16, device=A6.device)
+    if M and N:
+        _run("flh_gemm_f6_swiglu_o16", A6.device, A6.data_ptr(), B6_gate.data_ptr(), B6_up.data_ptr(), A_scale.data_ptr(),
+             gate_scale.data_ptr(), up_scale.data_ptr(), D.data_ptr(), M, N, K, A_scale.size(1), gate_scale.size(1),
+             _stream(A6))
+    return D
+
+
 def gemm_f6_dequant_multi(A6, B6s, A_scale, B_scales):
     """gemm_f6_dequant_o16 (all scales one column) resp. gemm_f6_dequant_o16_gs for up to four encoded weight
     matrices that share the encoded activations, in one launch -> list of fp16 [M, N_s], same bits as the single calls."""

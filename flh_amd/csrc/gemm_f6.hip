@@ -43,7 +43,12 @@ constexpr int kBf6 = 3;           // format selector of the matrix instruction: 
 
 typedef int v8i __attribute__((ext_vector_type(8)));
 
-template <int BM, int BN, int WM, int WN, int STAGES, int EPI>
+//
+// SWIGLU (as in the int8 kernel): the launch computes gate = A . Bg^T and up = A . Bu^T for the SAME output channels in one
+// workgroup -- the tile's BN weight rows are BN / 2 rows of the gate matrix and the same BN / 2 rows of the up matrix, the
+// two wave columns -- rounds both to fp16 as their own launches would store them, and stores only
+// fp16(fp16(silu(gate)) * up): [M, N] with N the width of ONE of the matrices.
+template <int BM, int BN, int WM, int WN, int STAGES, int EPI, bool SWIGLU = false>
 __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN), ((BM / WM) * (BN / WN) == 4 && WM * WN <= 64 * 64) ? 2 : 1)
 void gemm_f6_kernel(const GemmArgs p) {
   constexpr int TM = WM / 32, TN = WN / 32;
@@ -56,6 +61,8 @@ void gemm_f6_kernel(const GemmArgs p) {
   constexpr int NI = NI_LO + (NI_X ? 1 : 0);
   constexpr int EPI_PITCH = WN * 2 + kEpiPadF6;
   static_assert((WAVES == 4 || WAVES == 8) && BM % 64 == 0 && BN % 64 == 0, "tile shape");
+  static_assert(!SWIGLU || (EPI != kInt32 && WAVES_N == 2), "gate | up halves are the two wave columns");
+  constexpr int BNC = SWIGLU ? BN / 2 : BN;           // output channels per tile
   static_assert((BM + BN) * 6 % 64 == 0 && (BM * 6) % 64 == 0, "whole load instructions, none straddling A | B");
   static_assert(STAGES >= 3, "ring depth");
   static_assert(EPI == kInt32 || WAVES * WM * EPI_PITCH <= STAGES * STAGE, "epilogue staging must fit the ring");
@@ -93,22 +100,24 @@ void gemm_f6_kernel(const GemmArgs p) {
       wN = p.seg_N[s];
       seg_tile = tile_n - p.seg_tile0[s];
     }
-  const int m0 = tile_m * BM, n0 = seg_tile * BN;
+  const int m0 = tile_m * BM, n0 = seg_tile * BNC;
 
   // per-lane byte offsets of this wave's NI load instructions inside A resp. B (stage 0)
   const int my_ni = NI_LO + (wave < NI_X ? 1 : 0);     // wave-uniform
   const int first_i = wave * NI_LO + (wave < NI_X ? wave : NI_X);
   unsigned voff[NI];
-  bool from_a[NI];
+  int src_of[NI];                                      // 0: activations, 1: weights, 2: the up matrix (SWIGLU)
+  static_assert(!SWIGLU || (BNC * 6) % 64 == 0, "a load instruction never straddles gate | up");
 #pragma unroll
   for (int i = 0; i < NI; ++i) {
     const int slot = (min(first_i + i, TI - 1)) * 64 + lane;
     const bool isA = __builtin_amdgcn_readfirstlane(slot < BM * 6);
     const int s = isA ? slot : slot - BM * 6;
     const int r = s / 6, c = (s % 6) ^ ((r >> 3) & 1);
-    const int gr = isA ? min(m0 + r, p.M - 1) : min(n0 + r, wN - 1);
+    const bool second = SWIGLU && !isA && __builtin_amdgcn_readfirstlane(s >= BNC * 6);
+    const int gr = isA ? min(m0 + r, p.M - 1) : min(n0 + (second ? r - BNC : r), wN - 1);
     voff[i] = (unsigned)gr * kBlockBytes + c * 16;
-    from_a[i] = isA;
+    src_of[i] = isA ? 0 : second ? 2 : 1;
   }
   const int KT = p.K / 128;
   auto issue_stage = [&](int stage, int kt) {
@@ -116,9 +125,11 @@ void gemm_f6_kernel(const GemmArgs p) {
     const unsigned base = lds0 + stage * STAGE + first_i * 1024;
     const uint8_t* ka = p.A + (size_t)k * p.M * kBlockBytes;   // slab k of either operand
     const uint8_t* kb = wB + (size_t)k * wN * kBlockBytes;
+    const uint8_t* kb2 = SWIGLU ? p.B2 + (size_t)k * wN * kBlockBytes : kb;
 #pragma unroll
     for (int i = 0; i < NI; ++i)
-      if (i < NI_LO || i < my_ni) load_to_lds16(from_a[i] ? ka : kb, voff[i], base + i * 1024);
+      if (i < NI_LO || i < my_ni)
+        load_to_lds16(src_of[i] == 0 ? ka : src_of[i] == 1 ? kb : kb2, voff[i], base + i * 1024);
   };
   // wait until at most `stages` stages of this wave's loads are still in flight
   auto wait_stages = [&](auto stages_tag) {
@@ -179,8 +190,11 @@ void gemm_f6_kernel(const GemmArgs p) {
   unsigned short sraw[8];
   const bool sc_thread = tid < SCROWS;
   const int sc_cols = tid < BM ? p.a_cols : p.b_cols;
+  const int sc_brow = min(tid, SCROWS - 1) - BM;      // weight row of the tile this thread fetches scales for
+  const bool sc_second = SWIGLU && sc_brow >= BNC;
   const __half* const sc_src = (tid < BM ? p.As + (size_t)min(m0 + tid, p.M - 1) * p.a_cols
-                                         : wBs + (size_t)min(n0 + min(tid, SCROWS - 1) - BM, wN - 1) * p.b_cols);
+                                         : (sc_second ? p.Bs2 : wBs) +
+                                               (size_t)min(n0 + (sc_second ? sc_brow - BNC : sc_brow), wN - 1) * p.b_cols);
   auto sc_issue = [&](int blk) {
 #pragma unroll
     for (int i = 0; i < 8; ++i) sraw[i] = ((const unsigned short*)sc_src)[min(blk * 8 + i, sc_cols - 1)];
@@ -239,9 +253,10 @@ void gemm_f6_kernel(const GemmArgs p) {
 #pragma unroll
     for (int i = 0; i < (BM + BN + T - 1) / T; ++i) {
       const int e = tid + i * T;
-      const int m = m0 + e, n = n0 + e - BM;
+      const bool second = SWIGLU && e - BM >= BNC;
+      const int m = m0 + e, n = n0 + e - BM - (second ? BNC : 0);
       scale_reg[i] = e < BM ? (m < p.M ? p.As[m] : __float2half(1.f))
-                            : (e < BM + BN && n < wN ? wBs[n] : __float2half(1.f));
+                            : (e < BM + BN && n < wN ? (second ? p.Bs2 : wBs)[n] : __float2half(1.f));
     }
   }
   if constexpr (GROUPED) sc_issue(0);
@@ -357,10 +372,40 @@ void gemm_f6_kernel(const GemmArgs p) {
           *(h4*)(ep + (i * 32 + frag_row) * EPI_PITCH + nl * 2) = v;
         }
       }
-    // ... and write it out as whole row segments (the tile is private to the wave: no barrier)
     constexpr int CPR = WN / 8, RPI = 64 / CPR;
     const int crow = lane / CPR, cchunk = lane % CPR;
     const bool vec_ok = (wN & 7) == 0;
+    if constexpr (SWIGLU) {
+      // the gate tile (left wave column) and the up tile (right wave column) of this row band are both in LDS after
+      // the barrier; each of the two waves combines half of the band's rows and stores 16-byte runs of the product
+      __syncthreads();
+      const int wcol = wave % WAVES_N;
+      const uint8_t* gate_t = lds + (wave - wcol) * (WM * EPI_PITCH);
+      const uint8_t* up_t = gate_t + WM * EPI_PITCH;
+#pragma unroll
+      for (int it = 0; it < WM / (2 * RPI); ++it) {
+        const int row = wcol * (WM / 2) + it * RPI + crow;
+        const int m = m0 + wm + row, n = n0 + cchunk * 8;
+        const h8 g8 = *(const h8*)(gate_t + row * EPI_PITCH + cchunk * 16);
+        const h8 u8 = *(const h8*)(up_t + row * EPI_PITCH + cchunk * 16);
+        h8 o;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) o[e] = silu_mul_f16(g8[e], u8[e]);
+        if (m < p.M) {
+          __half* dst = (__half*)wD + (size_t)m * wN + n;
+          if (vec_ok && n + 8 <= wN) {
+            *(h8*)dst = o;
+          } else {
+            const __half* hv = (const __half*)&o;
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+              if (n + e < wN) dst[e] = hv[e];
+          }
+        }
+      }
+      return;
+    }
+    // ... and write it out as whole row segments (the tile is private to the wave: no barrier)
 #pragma unroll
     for (int it = 0; it < WM / RPI; ++it) {
       const int row = it * RPI + crow;
@@ -381,10 +426,11 @@ void gemm_f6_kernel(const GemmArgs p) {
   }
 }
 
-template <int BM, int BN, int WM, int WN, int STAGES, int EPI>
+template <int BM, int BN, int WM, int WN, int STAGES, int EPI, bool SWIGLU = false>
 int launch_f6(GemmArgs a, hipStream_t stream) {
+  constexpr int BNC = SWIGLU ? BN / 2 : BN;           // output channels per tile
   a.tiles_m = (a.M + BM - 1) / BM;
-  a.tiles_n = (a.N + BN - 1) / BN;
+  a.tiles_n = (a.N + BNC - 1) / BNC;
   for (int s = 1; s < a.n_seg; ++s) {                 // further weight matrices: their tiles follow
     a.seg_tile0[s] = a.tiles_n;
     a.tiles_n += (a.seg_N[s] + BN - 1) / BN;
@@ -392,7 +438,7 @@ int launch_f6(GemmArgs a, hipStream_t stream) {
   a.group_m = a.tiles_m < 4 ? a.tiles_m : 4;
   const size_t smem = (size_t)STAGES * (BM + BN) * kBlockBytes +
                       (EPI == kRowScale ? (BM + BN) * 2 : (EPI == kGroupScale || EPI == kTokenGroup) ? (BM + BN) * 32 : 0);
-  auto kern = gemm_f6_kernel<BM, BN, WM, WN, STAGES, EPI>;
+  auto kern = gemm_f6_kernel<BM, BN, WM, WN, STAGES, EPI, SWIGLU>;
   static std::atomic<bool> attr_set{false};   // set-up is idempotent: a race only repeats it  // per instantiation
   if (!attr_set.load(std::memory_order_acquire)) {
     if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess)
@@ -416,6 +462,17 @@ int launch_f6_grouped(const GemmArgs& a, hipStream_t stream) {
   auto tiles = [&](int bm, int bn) { return (long)((a.M + bm - 1) / bm) * ((n_all + bn - 1) / bn); };
   if (tiles(128, 128) >= 200) return launch_f6<128, 128, 64, 64, 3, EPI>(a, stream);
   return launch_f6<64, 64, 32, 32, 3, EPI>(a, stream);
+}
+
+// SwiGLU launches: tiles by the number of 64-channel output tiles (128 weight rows of [gate | up] each)
+template <int EPI>
+int launch_f6_swiglu(const GemmArgs& a, hipStream_t stream) {
+  auto tiles = [&](int bm, int bnc) { return (long)((a.M + bm - 1) / bm) * ((a.N + bnc - 1) / bnc); };
+  int tile = tiles(128, 64) >= 200 ? 128 : 64;
+  const int forced = g_tune_tile.load(std::memory_order_relaxed);
+  if (forced == 128 || forced == 64) tile = forced;
+  if (tile == 128) return launch_f6<128, 128, 64, 64, 3, EPI, true>(a, stream);
+  return launch_f6<64, 64, 32, 32, 3, EPI, true>(a, stream);
 }
 
 // flh_gemm_set_tuning overrides the tile choice (256 / 128 / 64; the hook through which the tests cover every variant)
@@ -507,6 +564,27 @@ extern "C" int flh_gemm_f6_o16_gs(const uint8_t* A6, const uint8_t* B6, const fl
   GemmArgs g{A6, B6, (const __half*)a_scale, (const __half*)b_scale, D, (int)M, (int)N, (int)K, a_cols, b_cols, 0, 0, 0};
   if (a_cols == 1) return launch_f6_grouped<kTokenGroup>(g, (hipStream_t)stream);
   return launch_f6_grouped<kGroupScale>(g, (hipStream_t)stream);
+}
+
+extern "C" int flh_gemm_f6_swiglu_o16(const uint8_t* A6, const uint8_t* B6_gate, const uint8_t* B6_up, const flh_half* a_scale,
+                                      const flh_half* gate_scale, const flh_half* up_scale, flh_half* D, size_t M, size_t N,
+                                      size_t K, int a_cols, int b_cols, void* stream) {
+  if (int e = check_f6(A6, B6_gate, D, M, N, K)) return e;
+  if ((M && N) && !B6_up) return fail(FLH_EINVAL, "gemm_f6: null pointer");
+  if (misaligned16(B6_up)) return fail(FLH_EINVAL, "gemm_f6: A, B and D must be 16-byte aligned");
+  if (M == 0 || N == 0) return FLH_OK;
+  if (!a_scale || !gate_scale || !up_scale) return fail(FLH_EINVAL, "gemm_f6: null scale pointer");
+  const int ng = (int)(K / 128);
+  const bool grouped = a_cols != 1 || b_cols != 1;
+  if (grouped && (b_cols != ng || (a_cols != 1 && a_cols != ng)))
+    return fail(FLH_EINVAL, "gemm_f6 (SwiGLU): scale columns (%d, %d): weights need 1 or K / 128 = %d, activations 1 or %d",
+                a_cols, b_cols, ng, ng);
+  GemmArgs g{A6, B6_gate, (const __half*)a_scale, (const __half*)gate_scale, D, (int)M, (int)N, (int)K, a_cols, b_cols, 0, 0, 0};
+  g.B2 = B6_up;
+  g.Bs2 = (const __half*)up_scale;
+  if (!grouped) return launch_f6_swiglu<kRowScale>(g, (hipStream_t)stream);
+  if (a_cols == 1) return launch_f6_swiglu<kTokenGroup>(g, (hipStream_t)stream);
+  return launch_f6_swiglu<kGroupScale>(g, (hipStream_t)stream);
 }
 
 extern "C" int flh_gemm_f6_o16_multi(const uint8_t* A6, const flh_half* a_scale, int count, const uint8_t* const* B6,

@@ -143,6 +143,15 @@ class LinearFLH(torch.nn.Module):
         rows = x.view(-1, x.size(-1))
         n, k = gate_layer.out_features, gate_layer.in_features
         group = gate_layer.weight_group_size if gate_layer.weight_group_size > 0 else (gate_layer.in_group_size or 128)
+        a_rows = a_scale.reshape(rows.size(0), -1)
+        encoded = rows.size(1) * 4 == k * 3                     # activations already in the 6-bit format
+        six = [l._six_bit_applies(rows, a_rows, l.w_scale.view(n, -1), group) for l in (gate_layer, up_layer)]
+        if encoded or all(six):
+            ops = _pkg._CUDA
+            a6 = rows.contiguous() if encoded else ops.encode_f6(rows.contiguous())
+            y = ops.gemm_f6_swiglu(a6, gate_layer._six_bit_weights(), up_layer._six_bit_weights(), a_rows.contiguous(),
+                                   gate_layer.w_scale.view(n, -1), up_layer.w_scale.view(n, -1))
+            return y.view(*lead, n)
         y = _pkg._CUDA.gemm_i4_swiglu(rows, gate_layer.w_packed.view(n, k // 2), up_layer.w_packed.view(n, k // 2),
                                       a_scale.reshape(rows.size(0), -1), gate_layer.w_scale.view(n, -1),
                                       up_layer.w_scale.view(n, -1), group)

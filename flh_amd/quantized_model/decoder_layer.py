@@ -371,11 +371,6 @@ class W4A4DecoderLayer(torch.nn.Module):
         cols = g.w_scale.view(g.out_features, -1).size(1)
         return g.bias is None and self.up_proj.bias is None and (cols == 1 or (g.weight_group_size == 128 and cols == g.in_features // 128))
 
-    def _six_bit_gate_up(self, n_rows):
-        """Whether gate / up take the 6-bit matrix instruction for this many rows (faster than the int8 launch that fuses
-        the SwiGLU product when the weights carry group scales)."""
-        return all(l.wants_six_bit(n_rows) for l in (self.gate_proj, self.up_proj))
-
     def _group_quant(self, stage, quantizer, x):
         s, z, q = quantizer(x)
         self._tap(stage + ".input", x.reshape(-1, x.size(-1)))
@@ -392,7 +387,7 @@ class W4A4DecoderLayer(torch.nn.Module):
                                                self.mlp_quantizer1, x, add, (self.gate_proj, self.up_proj))
         rows = q.numel() // q.size(-1)
         if (self.activation == "token" and self.fused and self.record is None and rows > 64
-                and self._swiglu_gemm_applies() and not self._six_bit_gate_up(rows)):
+                and self._swiglu_gemm_applies()):
             # prefill: gate and up in one launch that stores silu(gate) * up only (no fp16 [M, I] round trips)
             s, z, q = self._token_quant("mlp_mid", LinearFLH.forward_swiglu(self.gate_proj, self.up_proj, q, s),
                                         consumers=(self.down_proj,))

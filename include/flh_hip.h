@@ -193,6 +193,14 @@ int flh_gemm_f6_o16_multi(const uint8_t* A6, const flh_half* a_scale, int count,
                           const flh_half* const* b_scale, flh_half* const* D, const size_t* N, size_t M, size_t K,
                           int a_cols, int b_cols, void* stream);
 
+/* flh_gemm_i4_swiglu_o16 on 6-bit operands: gate = A . Bg^T and up = A . Bu^T in one launch that stores only
+ * D[m, n] = fp16(fp16(silu(gate)) * up), [M, N] with N the width of one of the two encoded weight matrices.  a_cols = b_cols
+ * = 1: one scale per row / channel; b_cols = K / 128 with a_cols 1 or K / 128: groups of 128.  Same bits as
+ * flh_gemm_i4_swiglu_o16 on the nibble operands. */
+int flh_gemm_f6_swiglu_o16(const uint8_t* A6, const uint8_t* B6_gate, const uint8_t* B6_up, const flh_half* a_scale,
+                           const flh_half* gate_scale, const flh_half* up_scale, flh_half* D, size_t M, size_t N, size_t K,
+                           int a_cols, int b_cols, void* stream);
+
 /* -------------------------------------------------------------------------------------
  * The two elementwise producers of quantised activations in a Llama block, fused into the group quantiser so
  * that the fp16 intermediate never goes to memory.  Neither has a native counterpart in the reference, which

@@ -119,3 +119,41 @@ def test_swiglu_layer_method_and_errors(ops):
         LinearFLH.forward_swiglu(gate, LinearFLH(k, n + 64, device="cuda"), dev(ap), dev(sa))
     with pytest.raises(RuntimeError):
         ops.gemm_i4_swiglu(dev(ap), dev(bg), dev(bu)[:-1], dev(sa), dev(sg), dev(su), 128)
+
+
+@pytest.mark.parametrize("m,n,k", [(300, 200, 512), (64, 64, 128), (513, 1000, 1024), (2048, 1408, 4096), (130, 36, 384)])
+@pytest.mark.parametrize("a_cols,b_cols", [(1, 1), (1, 2), (2, 2)])
+@pytest.mark.parametrize("tile", [0, 64, 128])
+def test_six_bit_swiglu_gemm_gives_the_int8_launch_bits(ops, gemm_tuning, m, n, k, a_cols, b_cols, tile):
+    """flh_gemm_f6_swiglu_o16 on re-encoded operands against flh_gemm_i4_swiglu_o16 on the nibbles: the sums are the same
+    integers, the epilogue the same arithmetic, the product the same device routine -- so bit for bit, for every scale
+    layout, ragged M and N, both tiles."""
+    print(f"case f6 swiglu m={m} n={n} k={k} a_cols={a_cols} b_cols={b_cols} tile={tile}", flush=True)
+    ap, bg, bu, sa, sg, su = case(m, n, k, 31 + m + n, a_cols, b_cols)
+    a, g, u = dev(ap), dev(bg), dev(bu)
+    want = ops.gemm_i4_swiglu(a, g, u, dev(sa), dev(sg), dev(su))
+    gemm_tuning(tile, 0)
+    got = ops.gemm_f6_swiglu(ops.encode_f6(a), ops.encode_f6(g), ops.encode_f6(u), dev(sa), dev(sg), dev(su))
+    gemm_tuning(0, 0)
+    assert got.shape == (m, n)
+    assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+    # ... and against the separate 6-bit launches followed by the product kernel
+    g6 = ops.gemm_f6_dequant_o16(ops.encode_f6(a), ops.encode_f6(g), dev(sa), dev(sg)) if b_cols == 1 else \
+        ops.gemm_f6_dequant_o16_gs(ops.encode_f6(a), ops.encode_f6(g), dev(sa), dev(sg))
+    u6 = ops.gemm_f6_dequant_o16(ops.encode_f6(a), ops.encode_f6(u), dev(sa), dev(su)) if b_cols == 1 else \
+        ops.gemm_f6_dequant_o16_gs(ops.encode_f6(a), ops.encode_f6(u), dev(sa), dev(su))
+    if n % 8 == 0:
+        assert torch.equal(got, ops.silu_mul(g6, u6))
+
+
+def test_six_bit_swiglu_argument_errors(ops):
+    a6 = torch.zeros(4, 96, dtype=torch.uint8, device="cuda")
+    b6 = torch.zeros(8, 96, dtype=torch.uint8, device="cuda")
+    s1 = torch.ones(4, 1, dtype=torch.float16, device="cuda")
+    w1 = torch.ones(8, 1, dtype=torch.float16, device="cuda")
+    with pytest.raises(RuntimeError):
+        ops.gemm_f6_swiglu(a6, b6, b6[:4].contiguous(), s1, w1, w1)
+    with pytest.raises(RuntimeError):
+        ops.gemm_f6_swiglu(a6, b6, b6, s1, w1, w1[:4].contiguous())
+    with pytest.raises(RuntimeError):
+        ops.gemm_f6_swiglu(a6, b6, b6, torch.ones(4, 3, dtype=torch.float16, device="cuda"), w1, w1)
