@@ -51,6 +51,29 @@ def test_argument_errors_come_back_before_any_launch():
         ("flh_rotate_quant_i4", (ok, ok, ok, odd, 4, 4096, 1, 0, 0, 1.0, st), b"16-byte aligned"),
         ("flh_group_quant_i4", (ok, odd, ok, 4, 128, 1, 1.0, st), b"16-byte aligned"),
         ("flh_fwht_f16_inplace", (odd, 4, 128, st), b"16-byte aligned"),
+        ("flh_gemm_i4_swiglu_o16", (ok, ok, odd, ok, ok, ok, ok, 16, 128, 128, 1, 1, 128, st), b"16-byte aligned"),
+        ("flh_gemm_i4_swiglu_o16", (ok, ok, ok, ok, ok, ok, ok, 16, 128, 192, 1, 1, 128, st), b"multiple of 128"),
+        ("flh_gemm_f6_o16", (ok, odd, ok, ok, ok, 16, 128, 128, st), b"16-byte aligned"),
+        ("flh_gemm_f6_o16_gs", (ok, ok, ok, ok, ok, 16, 128, 256, 3, 2, st), b"scale columns"),
+        ("flh_gemm_f6_swiglu_o16", (ok, ok, ok, ok, ok, ok, ok, 16, 128, 256, 2, 5, st), b"scale columns"),
+        ("flh_gemm_f6_i32", (ok, ok, ok, 16, 128, 100, st), b"multiple of 128"),
+        ("flh_encode_f6", (ok, ok, 4, 100, st), b"multiple of 128"),
+        ("flh_group_quant_f6", (odd, ok, ok, 4, 128, 1, 1.0, st), b"16-byte aligned"),
+        ("flh_rotate_quant_f6", (ok, None, None, 0, None, 1e-5, ok, ok, 4, 1000, 1, 1.0, st), b"K (1000)"),
+        ("flh_rotate_quant_f6", (ok, ok, None, 0, None, 1e-5, ok, ok, 4, 4096, 1, 1.0, st), b"come together"),
+        ("flh_silu_mul_group_quant_i4", (ok, odd, ok, ok, 4, 128, 1, 1.0, st), b"16-byte aligned"),
+        ("flh_rmsnorm_group_quant_i4", (ok, ok, ok, ok, 4, 100, 1e-5, 128, 1, 1.0, st), b"multiple of the group size"),
+        ("flh_rmsnorm_rotate_quant_i4", (ok, ok, 1e-5, ok, ok, None, 4, 1000, 1, 1.0, st), b"K (1000)"),
+        ("flh_add_rmsnorm_rotate_quant_i4", (ok, ok, ok, ok, 1e-5, ok, ok, 4, 4096, 1, 1.0, st), b"must not be x or add"),
+        ("flh_silu_mul_rotate_quant_i4", (ok, ok, ok, ok, 4, 4096, st), b"11008 or 14336"),
+        ("flh_silu_mul_rotate_quant_i4", (ok, ok, ok, ok, 1000, 11008, st), b"at most 256 rows"),
+        ("flh_silu_mul_f16", (ok, ok, ok, 12, st), b"multiple of 8"),
+        ("flh_rotate_quant_gemm_i4_o16", (ok, ok, ok, ok, 8, 128, 4096, 1, st), b"at most 4 tokens"),
+        ("flh_rotate_quant_gemm_i4_o16", (ok, ok, ok, ok, 2, 128, 2048, 1, st), b"not supported"),
+        ("flh_decode_attention_f16", (ok, ok, ok, ok, 1, 32, 8, 100, 16, 16, 1.0, ok, 1 << 20, st), b"head_dim"),
+        ("flh_decode_attention_f16", (ok, ok, ok, ok, 1, 32, 8, 128, 2048, 2048, 1.0, ok, 16, st), b"workspace"),
+        ("flh_decode_attention_f16_static", (ok, ok, ok, ok, 4096, 32, 8, 128, 8192, 8192, 1.0, st), b"static array"),
+        ("flh_gemm_set_tuning", (100, 0), b"tile must be"),
     ]
     for name, args, message in calls:
         rc = getattr(lib, name)(*args)
