@@ -21,6 +21,13 @@ _SIG = {
     "flh_init": (_c.c_int, []),
     "flh_gemm_i4_o16": (_c.c_int, [_PTR, _PTR, _PTR, _PTR, _PTR, _c.c_size_t, _c.c_size_t, _c.c_size_t,
                                    _c.c_int, _c.c_int, _c.c_int, _PTR]),
+    "flh_gemm_i4_add_o16": (_c.c_int, [_PTR, _PTR, _PTR, _PTR, _PTR, _PTR, _c.c_size_t, _c.c_size_t, _c.c_size_t,
+                                       _c.c_int, _c.c_int, _c.c_int, _PTR]),
+    "flh_gemm_f6_add_o16": (_c.c_int, [_PTR, _PTR, _PTR, _PTR, _PTR, _PTR, _c.c_size_t, _c.c_size_t, _c.c_size_t,
+                                       _c.c_int, _c.c_int, _PTR]),
+    "flh_gemm_i4_qkv_rope_o16": (_c.c_int, [_PTR, _PTR, _PTR, _PTR, _PTR, _PTR, _PTR, _PTR, _PTR, _PTR, _c.c_uint32,
+                                            _c.c_uint32, _c.c_uint32, _c.c_uint32, _c.c_uint32, _c.c_size_t, _c.c_int,
+                                            _c.c_int, _c.c_int, _PTR]),
     "flh_gemm_i4_swiglu_o16": (_c.c_int, [_PTR, _PTR, _PTR, _PTR, _PTR, _PTR, _PTR, _c.c_size_t, _c.c_size_t, _c.c_size_t,
                                           _c.c_int, _c.c_int, _c.c_int, _PTR]),
     "flh_gemm_f6_swiglu_o16": (_c.c_int, [_PTR, _PTR, _PTR, _PTR, _PTR, _PTR, _PTR, _c.c_size_t, _c.c_size_t, _c.c_size_t,

@@ -84,6 +84,35 @@ def _gemm_i4_dequant_checked(A, B, A_scale, B_scale, group_size):
     return D
 
 
+def _check_residual(residual, M, N, device, out):
+    _check(residual.is_cuda and residual.dtype == torch.float16 and residual.is_contiguous() and residual.device == device,
+           "the residual must be a contiguous float16 CUDA tensor on the operands' device")
+    _check(residual.numel() == M * N and residual.size(-1) == N, "the residual must have the shape of the output")
+    if out is not None:
+        _check(out.is_cuda and out.dtype == torch.float16 and out.is_contiguous() and out.device == device and
+               out.numel() == M * N and out.size(-1) == N, "out must be a contiguous float16 CUDA tensor of the output's shape")
+
+
+def gemm_i4_dequant_add(A, B, A_scale, B_scale, residual, group_size=128, out=None):
+    """fp16(residual + gemm_i4_dequant(A, B, A_scale, B_scale, group_size)) in one launch: the residual addition of a
+    decoder layer in the GEMM's epilogue (the GEMM's own fp16 rounding, then one fp16 addition -- the bits of the two
+    separate operations).  residual [M, N] (or [..., N] with M rows) fp16; `out` may be the residual itself (in-place
+    update of the residual stream) -> fp16 [M, N] (or `out`)."""
+    _check_gemm_inputs(A, B, A_scale, B_scale)
+    M, Kp = A.shape
+    N, K = B.size(0), Kp * 2
+    _check(A_scale.dim() == 2 and B_scale.dim() == 2, "scale must be 2D")
+    _check(A_scale.size(0) == M, "A_scale.shape[0] must equal M")
+    _check(B_scale.size(0) == N, "B_scale.shape[0] must equal N")
+    _check(K % 128 == 0, "K must be a multiple of 128")
+    _check_residual(residual, M, N, A.device, out)
+    D = out if out is not None else torch.empty((M, N), dtype=torch.float16, device=A.device)
+    if M and N:
+        _run("flh_gemm_i4_add_o16", A.device, A.data_ptr(), B.data_ptr(), A_scale.data_ptr(), B_scale.data_ptr(),
+             residual.data_ptr(), D.data_ptr(), M, N, K, A_scale.size(1), B_scale.size(1), int(group_size), _stream(A))
+    return D
+
+
 def gemm_i4_dequant_multi(A, Bs, A_scale, B_scales, group_size=128):
     """gemm_i4_dequant of the same activations against several weight matrices (q / k / v, gate / up) in one
     launch: Bs, B_scales are lists of up to four [N_s, K/2] / [N_s, 1 | K/g] tensors -> list of fp16 [M, N_s],
@@ -108,6 +137,50 @@ def gemm_i4_dequant_multi(A, Bs, A_scale, B_scales, group_size=128):
     _run("flh_gemm_i4_o16_multi", A.device, A.data_ptr(), A_scale.data_ptr(), n, ptrs(Bs), ptrs(B_scales), ptrs(Ds),
          sizes, M, K, A_scale.size(1), B_scales[0].size(1), int(group_size), _stream(A))
     return Ds
+
+
+def _check_rope_cache(M, batch, Bs, cos, sin, positions, k_cache, v_cache, device):
+    _check(batch > 0 and M % batch == 0, "the rows of A must be batch * T tokens")
+    T = M // batch
+    _check(Bs[0].size(0) % 128 == 0 and Bs[1].size(0) % 128 == 0 and Bs[1].size(0) == Bs[2].size(0),
+           "q / k / v must have whole heads of 128 channels, k and v the same number")
+    Hq, Hkv = Bs[0].size(0) // 128, Bs[1].size(0) // 128
+    for c in (cos, sin):
+        _check(c.is_cuda and c.dtype == torch.float16 and c.is_contiguous() and tuple(c.shape) == (T, 128) and c.device == device,
+               "cos / sin must be contiguous float16 CUDA tensors [T, 128]")
+    _check(positions.is_cuda and positions.dtype == torch.int64 and positions.is_contiguous() and positions.numel() == T
+           and positions.device == device, "positions must be a contiguous int64 CUDA tensor [T]")
+    for c in (k_cache, v_cache):
+        _check(c.is_cuda and c.dtype == torch.float16 and c.is_contiguous() and c.dim() == 4 and c.device == device and
+               c.size(0) == batch and c.size(1) == Hkv and c.size(3) == 128 and c.shape == k_cache.shape,
+               "the caches must be contiguous float16 CUDA tensors [batch, kv_heads, max_len, 128]")
+    return T, Hq, Hkv, k_cache.size(2)
+
+
+def gemm_i4_qkv_rope(A, A_scale, Bs, B_scales, cos, sin, positions, k_cache, v_cache, batch, group_size=128):
+    """The q / k / v projections with the rotary embedding and the cache write in the GEMM's epilogue: what
+    gemm_i4_dequant_multi(A, Bs, ...) followed by rope_kv_cache_ computes, same bits, in one launch.  A [batch * T, K/2]
+    packed codes, Bs = [q, k, v] weights with heads of 128 channels, cos / sin [T, 128], positions [T] int64 (cache slots),
+    k_cache / v_cache [batch, kv_heads, max_len, 128] (written in place) -> rotated queries [batch, T, heads, 128]."""
+    import ctypes
+    _check(len(Bs) == 3 and len(B_scales) == 3, "three weight matrices (q, k, v), one scale tensor each")
+    for B, B_scale in zip(Bs, B_scales):
+        _check_gemm_inputs(A, B, A_scale, B_scale)
+        _check(A_scale.dim() == 2 and B_scale.dim() == 2, "scale must be 2D")
+        _check(B_scale.size(0) == B.size(0) and B_scale.size(1) == B_scales[0].size(1), "B_scale shapes")
+        _check(B.device == A.device and B_scale.device == A.device, "tensors must be on one device")
+    M, Kp = A.shape
+    K = Kp * 2
+    _check(K % 128 == 0, "K must be a multiple of 128")
+    _check(A_scale.size(0) == M, "A_scale.shape[0] must equal M")
+    T, Hq, Hkv, max_len = _check_rope_cache(M, batch, Bs, cos, sin, positions, k_cache, v_cache, A.device)
+    q_out = torch.empty((batch, T, Hq, 128), dtype=torch.float16, device=A.device)
+    if M:
+        ptrs = lambda ts: (ctypes.c_void_p * 3)(*[t.data_ptr() for t in ts])
+        _run("flh_gemm_i4_qkv_rope_o16", A.device, A.data_ptr(), A_scale.data_ptr(), ptrs(Bs), ptrs(B_scales), cos.data_ptr(),
+             sin.data_ptr(), positions.data_ptr(), q_out.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), batch, T, Hq, Hkv,
+             max_len, K, A_scale.size(1), B_scales[0].size(1), int(group_size), _stream(A))
+    return q_out
 
 
 def gemm_i4_swiglu(A, B_gate, B_up, A_scale, gate_scale, up_scale, group_size=128):
@@ -335,6 +408,27 @@ def gemm_f6_dequant_o16_gs(A6, B6, A_scale, B_scale):
     if M and N:
         _run("flh_gemm_f6_o16_gs", A6.device, A6.data_ptr(), B6.data_ptr(), A_scale.data_ptr(), B_scale.data_ptr(),
              D.data_ptr(), M, N, K, A_scale.size(1), ng, _stream(A6))
+    return D
+
+
+def gemm_f6_dequant_add(A6, B6, A_scale, B_scale, residual, out=None):
+    """gemm_i4_dequant_add on operands encoded by encode_f6 (or written by rotate_and_quantize_f6): scales all one column, or
+    weight scales [N, K/128] with A_scale [M, 1] or [M, K/128].  Same bits."""
+    M, N, K = _check_f6(A6, B6)
+    ng = K // 128
+    _check(A_scale.is_cuda and B_scale.is_cuda and A_scale.dtype == torch.float16 and B_scale.dtype == torch.float16,
+           "scales must be float16 CUDA tensors")
+    _check(A_scale.is_contiguous() and B_scale.is_contiguous() and A_scale.dim() == 2 and B_scale.dim() == 2,
+           "scales must be contiguous and 2D")
+    _check(A_scale.size(0) == M and B_scale.size(0) == N, "one row of scales per row of A and of B expected")
+    _check((A_scale.size(1), B_scale.size(1)) in ((1, 1), (1, ng), (ng, ng)),
+           "scale columns must be (1, 1), (1, K/128) or (K/128, K/128)")
+    _check(A_scale.device == A6.device and B_scale.device == A6.device, "tensors must be on one device")
+    _check_residual(residual, M, N, A6.device, out)
+    D = out if out is not None else torch.empty((M, N), dtype=torch.float16, device=A6.device)
+    if M and N:
+        _run("flh_gemm_f6_add_o16", A6.device, A6.data_ptr(), B6.data_ptr(), A_scale.data_ptr(), B_scale.data_ptr(),
+             residual.data_ptr(), D.data_ptr(), M, N, K, A_scale.size(1), B_scale.size(1), _stream(A6))
     return D
 
 

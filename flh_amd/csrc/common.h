@@ -36,6 +36,18 @@ __device__ __forceinline__ float round_here(float v) {
   return v;
 }
 
+// eight fp16 additions (four packed pairs), each rounded once
+__device__ __forceinline__ v4i add_h8(v4i a, v4i b) {
+  v4i r;
+#pragma unroll
+  for (int d = 0; d < 4; ++d) {
+    const unsigned ua = (unsigned)a[d], ub = (unsigned)b[d];   // (scalar copies: a bit cast of a vector element miscompiles)
+    const h2 s2 = __builtin_bit_cast(h2, ua) + __builtin_bit_cast(h2, ub);
+    r[d] = (int)__builtin_bit_cast(unsigned, s2);
+  }
+  return r;
+}
+
 // fp16( float(fp16(silu(gate))) * float(up) ): the two roundings of torch's fp16 silu followed by its fp16 multiply
 // (the product the reference's MLP hands to the quantiser of down_proj, flh/quantized_model/modeling_llama.py:522-526);
 // silu in float32 as g * rcp(1 + exp(-g)) on the hardware exponential and reciprocal

@@ -413,13 +413,14 @@ void gemm_f6_kernel(const GemmArgs p) {
       const v4i v = *(const v4i*)(ep + row * EPI_PITCH + cchunk * 16);
       if (m < p.M) {
         __half* dst = (__half*)wD + (size_t)m * wN + n;
+        const __half* res = p.R ? p.R + (size_t)m * wN + n : nullptr;   // residual: read before the store (may be D)
         if (vec_ok && n + 8 <= wN) {
-          *(v4i*)dst = v;
+          *(v4i*)dst = res ? add_h8(v, *(const v4i*)res) : v;
         } else {
-          const __half* hv = (const __half*)&v;
+          const _Float16* hv = (const _Float16*)&v;
 #pragma unroll
           for (int e = 0; e < 8; ++e)
-            if (n + e < wN) dst[e] = hv[e];
+            if (n + e < wN) ((_Float16*)dst)[e] = res ? hv[e] + ((const _Float16*)res)[e] : hv[e];
         }
       }
     }
@@ -562,6 +563,25 @@ extern "C" int flh_gemm_f6_o16_gs(const uint8_t* A6, const uint8_t* B6, const fl
   if (b_cols != ng || (a_cols != 1 && a_cols != ng))
     return fail(FLH_EINVAL, "gemm_f6: scale columns (%d, %d) must be (1 or K/128, K/128) with K/128 = %d", a_cols, b_cols, ng);
   GemmArgs g{A6, B6, (const __half*)a_scale, (const __half*)b_scale, D, (int)M, (int)N, (int)K, a_cols, b_cols, 0, 0, 0};
+  if (a_cols == 1) return launch_f6_grouped<kTokenGroup>(g, (hipStream_t)stream);
+  return launch_f6_grouped<kGroupScale>(g, (hipStream_t)stream);
+}
+
+extern "C" int flh_gemm_f6_add_o16(const uint8_t* A6, const uint8_t* B6, const flh_half* a_scale, const flh_half* b_scale,
+                                   const flh_half* residual, flh_half* D, size_t M, size_t N, size_t K, int a_cols,
+                                   int b_cols, void* stream) {
+  if (int e = check_f6(A6, B6, D, M, N, K)) return e;
+  if (M == 0 || N == 0) return FLH_OK;
+  if (!a_scale || !b_scale) return fail(FLH_EINVAL, "gemm_f6: null scale pointer");
+  if (!residual) return fail(FLH_EINVAL, "gemm_f6 (residual): null pointer");
+  if (misaligned16(residual)) return fail(FLH_EINVAL, "gemm_f6 (residual): the residual must be 16-byte aligned");
+  const int ng = (int)(K / 128);
+  const bool rows_only = a_cols == 1 && b_cols == 1;
+  if (!rows_only && (b_cols != ng || (a_cols != 1 && a_cols != ng)))
+    return fail(FLH_EINVAL, "gemm_f6: scale columns (%d, %d) must be (1, 1) or (1 or K/128, K/128) with K/128 = %d", a_cols, b_cols, ng);
+  GemmArgs g{A6, B6, (const __half*)a_scale, (const __half*)b_scale, D, (int)M, (int)N, (int)K, a_cols, b_cols, 0, 0, 0};
+  g.R = (const __half*)residual;
+  if (rows_only) return launch_f6_by_shape<kRowScale>(g, (hipStream_t)stream);
   if (a_cols == 1) return launch_f6_grouped<kTokenGroup>(g, (hipStream_t)stream);
   return launch_f6_grouped<kGroupScale>(g, (hipStream_t)stream);
 }

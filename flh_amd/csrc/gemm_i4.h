@@ -34,6 +34,15 @@ struct GemmArgs {
   // SwiGLU launches (gate = B / Bs, up = B2 / Bs2, N = channels of each, D [M, N] = fp16(fp16(silu(gate)) * up))
   const uint8_t* B2;
   const __half* Bs2;
+  // q / k / v launches with the rotary embedding and the cache write in the epilogue (three segments q, k, v of heads of
+  // 128 channels; row m = b * rope_T + t): q -> D [M, N] rotated; k -> seg_D[1] = key cache [B, rope_hkv, rope_max_len,
+  // 128] at slot rope_pos[t], rotated; v -> seg_D[2] = value cache, as it is.  cos / sin [rope_T, 128].
+  const __half* rope_cos;
+  const __half* rope_sin;
+  const long long* rope_pos;
+  int rope_T, rope_max_len, rope_hkv;
+  // residual (single weight matrix, fp16 output): D = fp16(R + fp16(the launch's result)), R [M, N]; may be D itself
+  const __half* R;
 };
 
 // Small-M (decode) kernels: weight-streaming, split over K inside a workgroup.

@@ -91,7 +91,14 @@ __device__ __forceinline__ void interleave_hint() {
 // BN/2 rows of the up matrix, so the waves of the left half of the tile hold gate values and those of the right half
 // the matching up values; both halves go through the epilogue's fp16 staging tiles in LDS (rounded to fp16 exactly as
 // the two separate GEMMs would store them), where each wave then combines half of the rows.
-template <int BM, int BN, int WM, int WN, int STAGES, int EPI, int GROUP = 128, int KS = 1, bool SWIGLU = false>
+//
+// ROPE: a q / k / v launch (three weight matrices, heads of 128 channels = one tile column each) whose epilogue applies
+// the rotary embedding to the query and key heads and writes keys and values into their cache slots -- the arithmetic of
+// rope_kv_cache_kernel (rope_cache.hip) on the fp16 values the plain launch would have stored, so the same bits without
+// the pass over q, k and v that follows the GEMM otherwise.  The two halves of a head are the two wave columns, paired
+// through the staging tiles as for SWIGLU.
+template <int BM, int BN, int WM, int WN, int STAGES, int EPI, int GROUP = 128, int KS = 1, bool SWIGLU = false,
+          bool ROPE = false>
 __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN) * KS, (KS == 1 && WM * WN <= 128 * 64) ? FLH_GEMM_OCC : 1)
 void gemm_i4_kernel(const GemmArgs p) {
   constexpr bool GROUPED = EPI == kGroupScale || EPI == kTokenGroup;
@@ -109,6 +116,7 @@ void gemm_i4_kernel(const GemmArgs p) {
                 "epilogue staging must fit the ring");
   static_assert(KS == 1 || (!GROUPED && (KS - 1) * BM * BN * 4 <= KS * STAGES * STAGE), "K split");
   static_assert(!SWIGLU || (KS == 1 && EPI != kInt32 && BN / WN == 2), "gate | up halves are the two wave columns");
+  static_assert(!ROPE || (KS == 1 && EPI != kInt32 && BN == 128 && WN == 64 && !SWIGLU), "a tile column is one head of 128");
   constexpr int BNC = SWIGLU ? BN / 2 : BN;           // output channels per tile
   constexpr int ES = (KS == 2 && TM % 2 == 0) ? 2 : 1;   // quads that take part in the epilogue
   constexpr int TE = TM / ES;                            // 32-row blocks of a wave tile finished per quad
@@ -136,7 +144,7 @@ void gemm_i4_kernel(const GemmArgs p) {
   const uint8_t* wB = p.B;
   const __half* wBs = p.Bs;
   void* wD = p.D;
-  int wN = p.N, seg_tile = tile_n;
+  int wN = p.N, seg_tile = tile_n, seg = 0;
   for (int s = 1; s < p.n_seg; ++s)
     if (tile_n >= p.seg_tile0[s]) {
       wB = p.seg_B[s];
@@ -144,6 +152,7 @@ void gemm_i4_kernel(const GemmArgs p) {
       wD = p.seg_D[s];
       wN = p.seg_N[s];
       seg_tile = tile_n - p.seg_tile0[s];
+      seg = s;
     }
   const int m0 = tile_m * BM, n0 = seg_tile * BNC;
   const int Kb = p.K >> 1;                            // bytes per packed row
@@ -557,6 +566,74 @@ void gemm_i4_kernel(const GemmArgs p) {
           }
         }
       }
+    } else if constexpr (ROPE) {
+      // the tile's 128 columns are one head: its first 64 channels sit in the left wave column's staging tile, the other
+      // 64 in the right one's; each of the two waves finishes half of the band's rows, both halves of every row.
+      // First every row's table entries and cache slot are requested (one memory latency for all of them, overlapping
+      // the barrier), then the rows are rotated and stored.
+      constexpr int NIT = TE * 32 / (2 * RPI);
+      const int wcol = wave % WAVES_N;
+      const int head = seg_tile;
+      h8 c1[NIT], c2[NIT], s1[NIT], s2[NIT];
+      long long slot[NIT];
+      int bi[NIT];
+      {
+        const int m_first = m0 + wm + wcol * (TE * 16) + crow;
+        int b = m_first / p.rope_T, tt = m_first - b * p.rope_T;
+#pragma unroll
+        for (int it = 0; it < NIT; ++it) {
+          const int m = m_first + it * RPI;
+          const int tc = m < p.M ? tt : 0;               // rows past the end: any valid table row, nothing is stored
+          bi[it] = b;
+          slot[it] = seg == 0 ? 0 : p.rope_pos[tc];
+          if (seg < 2) {
+            const __half* ct = p.rope_cos + (size_t)tc * 128 + cchunk * 8;
+            const __half* st = p.rope_sin + (size_t)tc * 128 + cchunk * 8;
+            c1[it] = *(const h8*)ct, c2[it] = *(const h8*)(ct + 64), s1[it] = *(const h8*)st, s2[it] = *(const h8*)(st + 64);
+          }
+          tt += RPI;
+          while (tt >= p.rope_T) tt -= p.rope_T, ++b;
+        }
+      }
+      __syncthreads();
+      const uint8_t* lo_t = lds + (wave - wcol) * (TE * 32 * EPI_PITCH);
+      const uint8_t* hi_t = lo_t + TE * 32 * EPI_PITCH;
+#pragma unroll
+      for (int it = 0; it < NIT; ++it) {
+        const int row = wcol * (TE * 16) + it * RPI + crow;
+        const int m = m0 + wm + row;
+        h8 x1 = *(const h8*)(lo_t + row * EPI_PITCH + cchunk * 16);
+        h8 x2 = *(const h8*)(hi_t + row * EPI_PITCH + cchunk * 16);
+        if (m < p.M) {
+          bool in_range = true;
+          __half* dst;
+          if (seg == 0) {
+            dst = (__half*)wD + (size_t)m * wN + head * 128;
+          } else {
+            in_range = slot[it] >= 0 && slot[it] < (long long)p.rope_max_len;
+            dst = (__half*)wD +
+                  (((size_t)bi[it] * p.rope_hkv + head) * p.rope_max_len + (size_t)(in_range ? slot[it] : 0)) * 128;
+          }
+          if (seg < 2) {                                 // queries and keys: fp16(fp16(x cos) + fp16(rotate_half(x) sin))
+            h8 y1, y2;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+              const _Float16 a1 = (_Float16)round_here((float)x1[e] * (float)c1[it][e]);
+              const _Float16 r1 = (_Float16)round_here(-1.f * (float)x2[e] * (float)s1[it][e]);
+              y1[e] = (_Float16)round_here((float)a1 + (float)r1);
+              const _Float16 a2 = (_Float16)round_here((float)x2[e] * (float)c2[it][e]);
+              const _Float16 r2 = (_Float16)round_here(1.f * (float)x1[e] * (float)s2[it][e]);
+              y2[e] = (_Float16)round_here((float)a2 + (float)r2);
+            }
+            x1 = y1;
+            x2 = y2;
+          }
+          if (in_range) {
+            *(h8*)(dst + cchunk * 8) = x1;
+            *(h8*)(dst + 64 + cchunk * 8) = x2;
+          }
+        }
+      }
     } else {
     // ... and write it out as whole row segments (the tile is private to the wave: no barrier)
 #pragma unroll
@@ -566,13 +643,14 @@ void gemm_i4_kernel(const GemmArgs p) {
       const v4i v = *(const v4i*)(ep + row * EPI_PITCH + cchunk * 16);
       if (m < p.M) {
         __half* dst = (__half*)wD + (size_t)m * wN + n;
+        const __half* res = p.R ? p.R + (size_t)m * wN + n : nullptr;   // residual: read before the store (may be D)
         if (vec_ok && n + 8 <= wN) {
-          *(v4i*)dst = v;
+          *(v4i*)dst = res ? add_h8(v, *(const v4i*)res) : v;
         } else {
-          const __half* hv = (const __half*)&v;
+          const _Float16* hv = (const _Float16*)&v;
 #pragma unroll
           for (int e = 0; e < 8; ++e)
-            if (n + e < wN) dst[e] = hv[e];
+            if (n + e < wN) ((_Float16*)dst)[e] = res ? hv[e] + ((const _Float16*)res)[e] : hv[e];
         }
       }
     }
@@ -587,7 +665,8 @@ int total_n(const GemmArgs& a) {
   return n;
 }
 
-template <int BM, int BN, int WM, int WN, int STAGES, int EPI, int GROUP = 128, int KS = 1, bool SWIGLU = false>
+template <int BM, int BN, int WM, int WN, int STAGES, int EPI, int GROUP = 128, int KS = 1, bool SWIGLU = false,
+          bool ROPE = false>
 int launch(GemmArgs a, hipStream_t stream) {
   constexpr int BNC = SWIGLU ? BN / 2 : BN;           // output channels per tile
   a.tiles_m = (a.M + BM - 1) / BM;
@@ -600,7 +679,7 @@ int launch(GemmArgs a, hipStream_t stream) {
   // the ring(s), plus the tile's fp16 scales (one per row, or two blocks of eight groups per row)
   const size_t smem = (size_t)KS * STAGES * (BM + BN) * kStageBytes +
                       (EPI == kRowScale ? (BM + BN) * 2 : (EPI == kGroupScale || EPI == kTokenGroup) ? (BM + BN) * 32 : 0);
-  auto kern = gemm_i4_kernel<BM, BN, WM, WN, STAGES, EPI, GROUP, KS, SWIGLU>;
+  auto kern = gemm_i4_kernel<BM, BN, WM, WN, STAGES, EPI, GROUP, KS, SWIGLU, ROPE>;
   static std::atomic<bool> attr_set{false};   // set-up is idempotent: a race only repeats it  // per instantiation
   if (!attr_set.load(std::memory_order_acquire)) {
     if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess)
@@ -699,6 +778,19 @@ int launch_swiglu(const GemmArgs& a, int group, hipStream_t stream) {
   }
 }
 
+// q / k / v launches with the rotary embedding and the cache write in the epilogue: 128-column tiles only
+template <int EPI>
+int launch_qkv_rope(const GemmArgs& a, hipStream_t stream) {
+  const long tiles256 = (long)((a.M + 255) / 256) * (total_n(a) / 128);
+  int tile = tiles256 > 256 ? 256 : 128;
+  const int forced = g_tune_tile.load(std::memory_order_relaxed);
+  if (forced == 256 || forced == 128) tile = forced;
+  if constexpr (EPI == kRowScale) {                    // (the group epilogues have one thread per scale row: 128 x 128 only)
+    if (tile == 256) return launch<256, 128, 128, 64, FLH_GEMM_STAGES, EPI, 128, 1, false, true>(a, stream);
+  }
+  return launch<128, 128, 64, 64, 3, EPI, 128, 1, false, true>(a, stream);
+}
+
 int check_common(const void* A, const void* B, const void* D, size_t M, size_t N, size_t K) {
   if ((M && N) && (!A || !B || !D)) return fail(FLH_EINVAL, "gemm: null pointer");
   if (misaligned16(A, B, D)) return fail(FLH_EINVAL, "gemm: A, B and D must be 16-byte aligned");
@@ -743,6 +835,27 @@ extern "C" int flh_gemm_i4_o16(const uint8_t* A, const uint8_t* B, const flh_hal
   return gemm_dispatch(g, grouped ? kGroupScale : kRowScale, group, (hipStream_t)stream);
 }
 
+extern "C" int flh_gemm_i4_add_o16(const uint8_t* A, const uint8_t* B, const flh_half* a_scale, const flh_half* b_scale,
+                                   const flh_half* residual, flh_half* D, size_t M, size_t N, size_t K, int a_cols,
+                                   int b_cols, int group, void* stream) {
+  if (int e = check_common(A, B, D, M, N, K)) return e;
+  if (M == 0 || N == 0) return FLH_OK;
+  if (!a_scale || !b_scale) return fail(FLH_EINVAL, "gemm: null scale pointer");
+  if (!residual) return fail(FLH_EINVAL, "gemm (residual): null pointer");
+  if (misaligned16(residual)) return fail(FLH_EINVAL, "gemm (residual): the residual must be 16-byte aligned");
+  const bool grouped = a_cols != 1 || b_cols != 1;
+  if (grouped) {
+    if (group != 128 && group != 64 && group != 32)
+      return fail(FLH_EINVAL, "gemm: group size %d not supported (32, 64 or 128)", group);
+    const int ng = (int)(K / group);
+    if ((a_cols != 1 && a_cols != ng) || (b_cols != 1 && b_cols != ng))
+      return fail(FLH_EINVAL, "gemm: scale columns (%d, %d) must be 1 or K/group = %d", a_cols, b_cols, ng);
+  }
+  GemmArgs g{A, B, (const __half*)a_scale, (const __half*)b_scale, D, (int)M, (int)N, (int)K, a_cols, b_cols, 0, 0, 0};
+  g.R = (const __half*)residual;
+  return gemm_dispatch(g, grouped ? kGroupScale : kRowScale, group, (hipStream_t)stream);
+}
+
 extern "C" int flh_gemm_i4_swiglu_o16(const uint8_t* A, const uint8_t* B_gate, const uint8_t* B_up, const flh_half* a_scale,
                                       const flh_half* gate_scale, const flh_half* up_scale, flh_half* D, size_t M, size_t N,
                                       size_t K, int a_cols, int b_cols, int group, void* stream) {
@@ -764,6 +877,50 @@ extern "C" int flh_gemm_i4_swiglu_o16(const uint8_t* A, const uint8_t* B_gate, c
   if (!grouped) return launch_swiglu<kRowScale>(g, group, (hipStream_t)stream);
   if (a_cols == 1) return launch_swiglu<kTokenGroup>(g, group, (hipStream_t)stream);
   return launch_swiglu<kGroupScale>(g, group, (hipStream_t)stream);
+}
+
+extern "C" int flh_gemm_i4_qkv_rope_o16(const uint8_t* A, const flh_half* a_scale, const uint8_t* const* B,
+                                        const flh_half* const* b_scale, const flh_half* cos, const flh_half* sin,
+                                        const int64_t* positions, flh_half* q_out, flh_half* k_cache, flh_half* v_cache,
+                                        uint32_t batch, uint32_t T, uint32_t Hq, uint32_t Hkv, uint32_t max_len, size_t K,
+                                        int a_cols, int b_cols, int group, void* stream) {
+  if (!B || !b_scale) return fail(FLH_EINVAL, "gemm (q/k/v + rotary): null array");
+  if (Hq == 0 || Hkv == 0 || max_len == 0) return fail(FLH_EINVAL, "gemm (q/k/v + rotary): heads and cache length must be positive");
+  const size_t M = (size_t)batch * T;
+  const size_t N[3] = {(size_t)Hq * 128, (size_t)Hkv * 128, (size_t)Hkv * 128};
+  flh_half* const D[3] = {q_out, k_cache, v_cache};
+  for (int s = 0; s < 3; ++s) {
+    if (int e = check_common(A, B[s], D[s], M, N[s], K)) return e;
+    if (!b_scale[s]) return fail(FLH_EINVAL, "gemm: null scale pointer");
+  }
+  if (M == 0) return FLH_OK;
+  if (!a_scale || !cos || !sin || !positions) return fail(FLH_EINVAL, "gemm (q/k/v + rotary): null pointer");
+  if (misaligned16(cos, sin)) return fail(FLH_EINVAL, "gemm (q/k/v + rotary): cos and sin must be 16-byte aligned");
+  if ((uint64_t)batch * Hkv * max_len > (1ull << 40) / 128) return fail(FLH_EINVAL, "gemm (q/k/v + rotary): cache too large");
+  const bool grouped = a_cols != 1 || b_cols != 1;
+  if (grouped) {
+    if (group != 128) return fail(FLH_EINVAL, "gemm (q/k/v + rotary): group-scaled operands need groups of 128, not %d", group);
+    const int ng = (int)(K / 128);
+    if ((a_cols != 1 && a_cols != ng) || (b_cols != 1 && b_cols != ng))
+      return fail(FLH_EINVAL, "gemm: scale columns (%d, %d) must be 1 or K/group = %d", a_cols, b_cols, ng);
+  }
+  GemmArgs g{A, B[0], (const __half*)a_scale, (const __half*)b_scale[0], q_out, (int)M, (int)N[0], (int)K, a_cols, b_cols, 0, 0, 0};
+  g.n_seg = 3;
+  for (int s = 1; s < 3; ++s) {
+    g.seg_B[s] = B[s];
+    g.seg_Bs[s] = (const __half*)b_scale[s];
+    g.seg_D[s] = D[s];
+    g.seg_N[s] = (int)N[s];
+  }
+  g.rope_cos = (const __half*)cos;
+  g.rope_sin = (const __half*)sin;
+  g.rope_pos = (const long long*)positions;
+  g.rope_T = (int)T;
+  g.rope_max_len = (int)max_len;
+  g.rope_hkv = (int)Hkv;
+  if (!grouped) return launch_qkv_rope<kRowScale>(g, (hipStream_t)stream);
+  if (a_cols == 1 && b_cols > 1) return launch_qkv_rope<kTokenGroup>(g, (hipStream_t)stream);
+  return launch_qkv_rope<kGroupScale>(g, (hipStream_t)stream);
 }
 
 extern "C" int flh_gemm_i4_o16_multi(const uint8_t* A, const flh_half* a_scale, int count, const uint8_t* const* B,

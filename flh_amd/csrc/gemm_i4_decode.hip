@@ -57,6 +57,13 @@ int decode_blocks(GemmArgs& a) {
   return blocks;
 }
 
+// one fp16 output; with a residual (single weight matrix) the stored value is fp16(R + value)
+__device__ __forceinline__ void store_f16(const GemmArgs& p, const DecodeWeights& w, int gm, int gn, _Float16 v) {
+  const size_t at = (size_t)gm * w.N + gn;
+  if (p.R) v = v + ((const _Float16*)p.R)[at];
+  ((_Float16*)w.D)[at] = v;
+}
+
 // Partial sums in LDS -> outputs.  Lane l of a tile holds token l % 16 and channels 4 (l / 16) + i, i = 0..3.
 // a_scales: one scale per token (row-scale epilogue); sA / sB: the group tables (group epilogue).
 template <int MT, int EPI>
@@ -78,7 +85,7 @@ __device__ __forceinline__ void decode_finish(const GemmArgs& p, const DecodeWei
         for (int g = 0; g < KT; ++g)
           out = __builtin_fmaf((float)(red[(g * MT + mt) * 256 + pos] >> 8), sA[g * 16 + m] * sB[g * 16 + n], out);
       }
-      ((__half*)w.D)[(size_t)gm * w.N + gn] = __float2half(round_here(out));
+      store_f16(p, w, gm, gn, (_Float16)round_here(out));
     } else {
       int sum = 0;
 #pragma unroll
@@ -88,7 +95,7 @@ __device__ __forceinline__ void decode_finish(const GemmArgs& p, const DecodeWei
       } else {
         // sum = 256 * (exact contraction); the weight scale carries the matching exact 2^-8
         const float sa = __half2float(a_scales[gm]), sb = __half2float(w.Bs[gn]) * 0.00390625f;
-        ((__half*)w.D)[(size_t)gm * w.N + gn] = __float2half(round_here((float)sum * (sa * sb)));
+        store_f16(p, w, gm, gn, (_Float16)round_here((float)sum * (sa * sb)));
       }
     }
   }

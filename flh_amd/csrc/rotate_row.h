@@ -71,18 +71,6 @@ __device__ __forceinline__ void stage_swap(float (&v)[N]) {
   }
 }
 
-// eight fp16 additions (four packed pairs), each rounded once
-__device__ __forceinline__ v4i add_h8(v4i a, v4i b) {
-  v4i r;
-#pragma unroll
-  for (int d = 0; d < 4; ++d) {
-    const unsigned ua = (unsigned)a[d], ub = (unsigned)b[d];   // (scalar copies: a bit cast of a vector element miscompiles)
-    const h2 s2 = __builtin_bit_cast(h2, ua) + __builtin_bit_cast(h2, ub);
-    r[d] = (int)__builtin_bit_cast(unsigned, s2);
-  }
-  return r;
-}
-
 // RMS: the row is first normalised as flh/nn/normalization.py:12-20 does -- float32 sum of squares / K,
 // x * (1 / sqrt(. + eps)) [* weight] with every product rounded to float32, then fp16 -- and that fp16 row is
 // what the rotation and the quantiser see.

@@ -73,10 +73,15 @@ class LinearFLH(torch.nn.Module):
         return grouped or (per_row and self.six_bit is True)
 
     # ------------------------------------------------------------------ kernels
-    def forward(self, x, a_scale=None, a_zero=None, x_is_packed=False, is_symmetric=None):
+    def forward(self, x, a_scale=None, a_zero=None, x_is_packed=False, is_symmetric=None, residual=None):
         """x: packed int4 activations [..., K/2] uint8; a_scale [..., K/in_group] or [..., 1]
-        fp16 (as returned by ActQuantizer).  Returns fp16 [..., N]."""
+        fp16 (as returned by ActQuantizer).  Returns fp16 [..., N].  `residual` (extension; fp16 [..., N]): returns
+        residual + forward(x, ...) from the same launch -- the layer output rounded to fp16 as always, then one fp16
+        addition in the GEMM's epilogue instead of a separate pass over both tensors."""
         lead = x.shape[:-1]
+        if residual is not None and self.bias is not None:
+            return residual + self.forward(x, a_scale, a_zero, x_is_packed, is_symmetric)
+        res = None if residual is None else residual.reshape(-1, self.out_features)
         rows = x.view(-1, x.size(-1))
         w_scale = self.w_scale.view(self.out_features, -1)
         group = self.weight_group_size if self.weight_group_size > 0 else (self.in_group_size or 128)
@@ -89,12 +94,18 @@ class LinearFLH(torch.nn.Module):
             if encoded and not ((w_scale.size(1) == 1 and a_rows.size(1) == 1) or
                                 (group == 128 and w_scale.size(1) == self.in_features // 128)):
                 raise ValueError("6-bit activations need per-token x per-channel scales or group-of-128 weight scales")
-            if w_scale.size(1) == 1:
+            if res is not None:
+                y = ops.gemm_f6_dequant_add(a6, w6, a_rows.contiguous(), w_scale, res.contiguous())
+            elif w_scale.size(1) == 1:
                 y = ops.gemm_f6_dequant_o16(a6, w6, a_rows.contiguous(), w_scale)
             else:
                 y = ops.gemm_f6_dequant_o16_gs(a6, w6, a_rows.contiguous(), w_scale)
             if self.bias is not None:
                 y = y + self.bias
+            return y.view(*lead, self.out_features)
+        if res is not None:
+            y = _pkg._CUDA.gemm_i4_dequant_add(rows, self.w_packed.view(self.out_features, self.in_features // 2),
+                                               a_rows, w_scale, res.contiguous(), group)
             return y.view(*lead, self.out_features)
         y = _pkg._CUDA.gemm_i4_dequant(rows, self.w_packed.view(self.out_features, self.in_features // 2),
                                        a_scale.reshape(rows.size(0), -1), w_scale, group)

@@ -266,11 +266,13 @@ class W4A4DecoderLayer(torch.nn.Module):
         kv_cache: None, a pair (keys, values) [B, kv_heads, past, head_dim] that grows by concatenation, or one layer
         of a StaticKVCache together with `positions` (device int64 [T]: the slots the new tokens take; the cache's
         kv_len says how many slots attention reads).  Causal over past + T positions."""
-        _, y, cache = self._attention(x, None, cos, sin, kv_cache, positions)
+        _, y, cache = self._attention(x, None, cos, sin, kv_cache, positions, fold_residual=False)
         return y, cache
 
-    def _attention(self, x, add, cos, sin, kv_cache=None, positions=None):
-        """attention() on the residual stream x + add (add may be None); returns that sum as well."""
+    def _attention(self, x, add, cos, sin, kv_cache=None, positions=None, fold_residual=True):
+        """attention() on the residual stream x + add (add may be None): returns (that sum, the attention block's output,
+        cache) -- or, when o_proj adds the residual in its epilogue (`fold_residual`, prefill sizes), (the stream after the
+        block, None, cache)."""
         b, t, _ = x.shape
         if (self.activation == "token" and self.fused and self.record is None and b * t <= 2 and self.hidden_size == 4096
                 and self._online_qkv_applies()):
@@ -286,6 +288,8 @@ class W4A4DecoderLayer(torch.nn.Module):
         else:
             x, s, z, q = self._residual_norm_quant("attn_in", self.input_layernorm, "input_layernorm",
                                                    self.attn_quantizer1, x, add, (self.q_proj, self.k_proj, self.v_proj))
+            if self._qkv_rope_applies(b * t, q, s, cos, kv_cache, positions):
+                return self._attention_after_fused_qkv(x, q, s, cos, sin, kv_cache, positions, fold_residual)
             qs, ks, vs = self._project([self.q_proj, self.k_proj, self.v_proj], q, s, z)
         self._tap("q_proj", qs), self._tap("k_proj", ks), self._tap("v_proj", vs)
         static = isinstance(kv_cache, StaticKVCache._Layer)
@@ -351,11 +355,79 @@ class W4A4DecoderLayer(torch.nn.Module):
                 and self.hidden_size == 4096):
             # decode: the quantiser runs inside the GEMM's own launch (same bits as the two launches)
             return x, self.o_proj.forward_online(out, hadamard="exact"), cache
+        return self._output_projection(x, out, cache, fold_residual)
+
+    def _output_projection(self, x, out, cache, fold_residual):
+        """quantiser + o_proj on the attention output `out` [B, T, hidden]; (stream, block output or None, cache) as
+        _attention returns them."""
         s, z, q = (self._token_quant("attn_out", out, consumers=(self.o_proj,)) if self.activation == "token"
                    else self._group_quant("attn_out", self.attn_quantizer2, out))
+        if fold_residual and self._residual_in_gemm(out.numel() // out.size(-1)):
+            # prefill: the residual addition in o_proj's epilogue; nothing is left pending
+            return self.o_proj(q, s, z, x_is_packed=True, residual=x), None, cache
         y = self.o_proj(q, s, z, x_is_packed=True)
         self._tap("o_proj", y)
         return x, y, cache
+
+    def _qkv_rope_applies(self, rows, codes, scales, cos, kv_cache, positions):
+        """Whether q / k / v take the launch whose epilogue applies the rotary embedding and writes the cache: the fused
+        prefill path with heads of 128 channels, nibble codes that stay on the int8 kernel (not the 6-bit format, no layer
+        that would re-encode them) and fp16 tables."""
+        static = isinstance(kv_cache, StaticKVCache._Layer)
+        layers = (self.q_proj, self.k_proj, self.v_proj)
+        group = self.q_proj.weight_group_size if self.q_proj.weight_group_size > 0 else (self.q_proj.in_group_size or 128)
+        if codes.size(-1) * 2 == self.hidden_size and all(
+                l._six_bit_applies(codes.reshape(rows, -1), scales.reshape(rows, -1), l.w_scale.view(l.out_features, -1), group)
+                for l in layers):
+            return False
+        return (self.fused and self.record is None and rows > 64 and rows > codes.size(0) and self.head_dim == 128 and codes.is_cuda
+                and codes.size(-1) * 2 == self.hidden_size and self._online_qkv_applies()
+                and cos.dtype == torch.float16 and tuple(cos.shape) == (rows // codes.size(0), 128)
+                and (positions is not None if static else True))
+
+    def _attention_after_fused_qkv(self, x, codes, scales, cos, sin, kv_cache, positions, fold_residual):
+        """The prefill attention block from the quantised input on: q / k / v, rotary embedding and cache write in one
+        launch (the bits of the separate launches), torch's fused attention, then the output projection."""
+        b, t, _ = x.shape
+        layers = [self.q_proj, self.k_proj, self.v_proj]
+        static = isinstance(kv_cache, StaticKVCache._Layer)
+        if static:
+            keys, values = kv_cache.tensors()
+            slots, cache = positions, kv_cache
+            past = None
+        else:
+            past = 0 if kv_cache is None else kv_cache[0].size(2)
+            keys = torch.empty(b, self.num_kv_heads, past + t, self.head_dim, dtype=x.dtype, device=x.device)
+            values = torch.empty_like(keys)
+            if past:
+                keys[:, :, :past] = kv_cache[0]
+                values[:, :, :past] = kv_cache[1]
+            slots = torch.arange(past, past + t, device=x.device)
+            cache = (keys, values)
+        group = self.q_proj.weight_group_size if self.q_proj.weight_group_size > 0 else (self.q_proj.in_group_size or 128)
+        qs = _ops().gemm_i4_qkv_rope(codes.reshape(b * t, -1), scales.reshape(b * t, -1),
+                                     [l.w_packed.view(l.out_features, l.in_features // 2) for l in layers],
+                                     [l.w_scale.view(l.out_features, -1) for l in layers], cos.contiguous(),
+                                     sin.contiguous(), slots, keys, values, b, group).transpose(1, 2)
+        if static:
+            n = kv_cache.owner.kv_len
+            keys, values = keys[:, :, :n], values[:, :, :n]
+            past = n - t
+        gqa = self.num_heads != self.num_kv_heads
+        if past == 0:
+            out = torch.nn.functional.scaled_dot_product_attention(qs, keys, values, is_causal=t > 1, enable_gqa=gqa)
+        else:
+            mask = torch.ones(t, past + t, dtype=torch.bool, device=x.device).tril(diagonal=past)
+            out = torch.nn.functional.scaled_dot_product_attention(qs, keys, values, attn_mask=mask, enable_gqa=gqa)
+        out = out.transpose(1, 2).reshape(b, t, self.hidden_size).contiguous()
+        return self._output_projection(x, out, cache, fold_residual)
+
+    def _residual_in_gemm(self, rows):
+        """Whether o_proj / down_proj add the residual stream in their own epilogue: the fused prefill path of the group
+        configuration, whose norm + quantiser launch has no addition of its own (measured at 2048 tokens: 728 against
+        736 us per layer).  The token configuration keeps the addition inside its norm + rotation launch, which is cheaper
+        than the extra read in the GEMM's epilogue burst (8 x 512 tokens: 888 against 910 us)."""
+        return self.fused and self.record is None and rows > 64 and self.activation == "group"
 
     def _online_qkv_applies(self):
         """q / k / v in the layout the decode GEMM with its own norm + quantiser takes: no bias, one scale per channel or
@@ -379,10 +451,11 @@ class W4A4DecoderLayer(torch.nn.Module):
         return s, z, q
 
     def mlp(self, x):
-        return self._mlp(x, None)[1]
+        return self._mlp(x, None, fold_residual=False)[1]
 
-    def _mlp(self, x, add):
-        """mlp() on the residual stream x + add (add may be None); returns (that sum, the MLP's output)."""
+    def _mlp(self, x, add, fold_residual=True):
+        """mlp() on the residual stream x + add (add may be None); returns (that sum, the MLP's output) -- or (the stream
+        after the block, None) when down_proj adds the residual in its epilogue (`fold_residual`, prefill sizes)."""
         x, s, z, q = self._residual_norm_quant("mlp_in", self.post_attention_layernorm, "post_attention_layernorm",
                                                self.mlp_quantizer1, x, add, (self.gate_proj, self.up_proj))
         rows = q.numel() // q.size(-1)
@@ -391,6 +464,8 @@ class W4A4DecoderLayer(torch.nn.Module):
             # prefill: gate and up in one launch that stores silu(gate) * up only (no fp16 [M, I] round trips)
             s, z, q = self._token_quant("mlp_mid", LinearFLH.forward_swiglu(self.gate_proj, self.up_proj, q, s),
                                         consumers=(self.down_proj,))
+            if fold_residual:
+                return self.down_proj(q, s, z, x_is_packed=True, residual=x), None
             return x, self.down_proj(q, s, z, x_is_packed=True)
         gate, up = self._project([self.gate_proj, self.up_proj], q, s, z)
         self._tap("gate_proj", gate), self._tap("up_proj", up)
@@ -407,18 +482,22 @@ class W4A4DecoderLayer(torch.nn.Module):
             s, z, q = self._silu_mul_quant(gate, up)
         else:
             s, z, q = self._group_quant("mlp_mid", self.mlp_quantizer2, torch.nn.functional.silu(gate) * up)
+        if fold_residual and self._residual_in_gemm(rows):
+            return self.down_proj(q, s, z, x_is_packed=True, residual=x), None
         y = self.down_proj(q, s, z, x_is_packed=True)
         self._tap("down_proj", y)
         return x, y
 
     def forward(self, x, cos, sin, kv_cache=None, positions=None):
         x, pending, cache = self.forward_deferred(x, None, cos, sin, kv_cache, positions)
-        return x + pending, cache
+        return (x if pending is None else x + pending), cache
 
     def forward_deferred(self, x, pending, cos, sin, kv_cache=None, positions=None):
         """The layer on the residual stream x + pending, with its own last addition left to the caller: returns
-        (stream, pending, cache) with the layer's output = stream + pending.  A stack of layers passes the pair on, so that
-        every residual addition runs inside the launch of the norm + quantiser that reads its result."""
+        (stream, pending, cache) with the layer's output = stream + pending (pending None: nothing left to add).  A stack
+        of layers passes the pair on, so that every residual addition runs inside another launch: for a few tokens that
+        of the norm + quantiser that reads its result, at prefill sizes the epilogue of the GEMM that produces the
+        addend."""
         x, attn, cache = self._attention(x, pending, cos, sin, kv_cache, positions)
         x, y = self._mlp(x, attn)
         return x, y, cache

@@ -61,6 +61,14 @@ int flh_gemm_i4_o16(const uint8_t* A, const uint8_t* B, const flh_half* a_scale,
                     flh_half* D, size_t M, size_t N, size_t K, int a_cols, int b_cols, int group,
                     void* stream);
 
+/* flh_gemm_i4_o16 with the residual addition of a decoder layer in its epilogue: D = fp16(residual + fp16(result)), the
+ * bits of the GEMM's own fp16 output followed by an fp16 addition (hidden = residual + o_proj(...) resp. + down_proj(...),
+ * flh/quantized_model/modeling_llama.py:600-618).  residual [M, N] fp16, 16-byte aligned; it may be D (in-place update of
+ * the residual stream).  No native counterpart in the reference, which adds in torch. */
+int flh_gemm_i4_add_o16(const uint8_t* A, const uint8_t* B, const flh_half* a_scale, const flh_half* b_scale,
+                        const flh_half* residual, flh_half* D, size_t M, size_t N, size_t K, int a_cols, int b_cols,
+                        int group, void* stream);
+
 /* flh_gemm_i4_o16 for several weight matrices that share the activations -- q / k / v, gate / up -- in ONE launch:
  * D[s] [M, N[s]] = the result of flh_gemm_i4_o16(A, B[s], a_scale, b_scale[s], ...) for s < count <= 4, same bits.
  * B, b_scale, D and N are host arrays of `count` entries (device pointers resp. sizes); a_cols, b_cols and group
@@ -71,6 +79,20 @@ int flh_gemm_i4_o16(const uint8_t* A, const uint8_t* B, const flh_half* a_scale,
 int flh_gemm_i4_o16_multi(const uint8_t* A, const flh_half* a_scale, int count, const uint8_t* const* B,
                           const flh_half* const* b_scale, flh_half* const* D, const size_t* N, size_t M, size_t K,
                           int a_cols, int b_cols, int group, void* stream);
+
+/* The q / k / v projections of an attention block in one launch whose epilogue applies the rotary embedding and writes the
+ * key / value cache: flh_gemm_i4_o16_multi (three weight matrices B[0..2] = q, k, v with Hq, Hkv, Hkv heads of 128 channels,
+ * scales b_scale[0..2]) followed by flh_rope_kv_cache_f16, same bits, without the pass over q, k and v in between
+ * (flh/quantized_model/modeling_llama.py:386-424 computes the three projections, transformers' apply_rotary_pos_emb and the
+ * cache update as separate tensor operations).  Rows of A are tokens b * T + t; cos, sin [T, 128] and positions [T] (int64,
+ * on the device) as in flh_rope_kv_cache_f16; q_out [batch, T, Hq, 128] receives the rotated queries, k_cache / v_cache
+ * [batch, Hkv, max_len, 128] the rotated keys resp. the values at slot positions[t] (a position outside the cache writes
+ * nothing).  Scales as in flh_gemm_i4_o16 (groups of 128 only). */
+int flh_gemm_i4_qkv_rope_o16(const uint8_t* A, const flh_half* a_scale, const uint8_t* const* B,
+                             const flh_half* const* b_scale, const flh_half* cos, const flh_half* sin,
+                             const int64_t* positions, flh_half* q_out, flh_half* k_cache, flh_half* v_cache,
+                             uint32_t batch, uint32_t T, uint32_t Hq, uint32_t Hkv, uint32_t max_len, size_t K,
+                             int a_cols, int b_cols, int group, void* stream);
 
 /* The gate and up projections of a SwiGLU MLP in one launch that stores only their combination:
  *   D[m, c] = fp16( float(fp16(silu(gate[m, c]))) * float(up[m, c]) ),  silu(g) = g / (1 + exp(-g)) in float32,
@@ -192,6 +214,11 @@ int flh_gemm_f6_o16_gs(const uint8_t* A6, const uint8_t* B6, const flh_half* a_s
 int flh_gemm_f6_o16_multi(const uint8_t* A6, const flh_half* a_scale, int count, const uint8_t* const* B6,
                           const flh_half* const* b_scale, flh_half* const* D, const size_t* N, size_t M, size_t K,
                           int a_cols, int b_cols, void* stream);
+
+/* flh_gemm_i4_add_o16 on 6-bit operands (a_cols = b_cols = 1, or groups of 128 as in flh_gemm_f6_o16_gs); same bits. */
+int flh_gemm_f6_add_o16(const uint8_t* A6, const uint8_t* B6, const flh_half* a_scale, const flh_half* b_scale,
+                        const flh_half* residual, flh_half* D, size_t M, size_t N, size_t K, int a_cols, int b_cols,
+                        void* stream);
 
 /* flh_gemm_i4_swiglu_o16 on 6-bit operands: gate = A . Bg^T and up = A . Bu^T in one launch that stores only
  * D[m, n] = fp16(fp16(silu(gate)) * up), [M, N] with N the width of one of the two encoded weight matrices.  a_cols = b_cols

@@ -74,11 +74,23 @@ def test_argument_errors_come_back_before_any_launch():
         ("flh_decode_attention_f16", (ok, ok, ok, ok, 1, 32, 8, 128, 2048, 2048, 1.0, ok, 16, st), b"workspace"),
         ("flh_decode_attention_f16_static", (ok, ok, ok, ok, 4096, 32, 8, 128, 8192, 8192, 1.0, st), b"static array"),
         ("flh_gemm_set_tuning", (100, 0), b"tile must be"),
+        ("flh_gemm_i4_add_o16", (ok, ok, ok, ok, odd, ok, 16, 128, 128, 1, 1, 128, st), b"residual must be 16-byte aligned"),
+        ("flh_gemm_i4_add_o16", (ok, ok, ok, ok, None, ok, 16, 128, 128, 1, 1, 128, st), b"null pointer"),
+        ("flh_gemm_f6_add_o16", (ok, ok, ok, ok, ok, ok, 16, 128, 256, 3, 2, st), b"scale columns"),
     ]
     for name, args, message in calls:
         rc = getattr(lib, name)(*args)
         assert rc == -1, (name, args, rc)                       # FLH_EINVAL
         assert message in lib.flh_last_error(), (name, lib.flh_last_error())
+    # the q / k / v launch with the rotary epilogue takes its three weight matrices and scales as pointer arrays
+    import ctypes
+    three = (ctypes.c_void_p * 3)(ok, ok, ok)
+    rope = lambda **kw: lib.flh_gemm_i4_qkv_rope_o16(
+        ok, ok, three, three, kw.get("cos", ok), ok, ok, ok, ok, ok, 2, 40, 4, kw.get("hkv", 2), 64, kw.get("k", 256),
+        1, kw.get("b_cols", 1), kw.get("group", 128), st)
+    for kw, message in (({"k": 192}, b"multiple of 128"), ({"hkv": 0}, b"must be positive"), ({"cos": odd}, b"16-byte aligned"),
+                        ({"b_cols": 2, "group": 64}, b"groups of 128")):
+        assert rope(**kw) == -1 and message in lib.flh_last_error(), (kw, lib.flh_last_error())
 
 
 def test_ops_fail_loudly_without_library(monkeypatch, tmp_path):
