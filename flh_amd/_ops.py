@@ -518,6 +518,29 @@ def rope_kv_cache_(q, k, v, cos, sin, positions, k_cache, v_cache):
 _attention_workspaces = {}      # (device index, stream handle) -> uint8 tensor: launches of one stream run in order
 
 
+def prefill_attention(q, k_cache, v_cache, past, scale=None):
+    """Causal attention of a block of T new tokens over a cache: q [B, T, Hq, 128] fp16 (token-major), k_cache / v_cache
+    [B, Hkv, max_len, 128] fp16 whose slots past .. past + T - 1 hold the block's own keys / values; query t sees the
+    slots 0 .. past + t.  -> [B, T, Hq * 128] fp16 = softmax(q K^T * scale) V, float32 softmax and accumulation,
+    probabilities rounded to fp16; grouped queries (Hq a multiple of Hkv)."""
+    for t_ in (q, k_cache, v_cache):
+        _check(t_.is_cuda and t_.dtype == torch.float16 and t_.is_contiguous() and t_.device == q.device,
+               "tensors must be contiguous float16 CUDA tensors on one device")
+    _check(q.dim() == 4 and k_cache.dim() == 4 and k_cache.shape == v_cache.shape and k_cache.size(0) == q.size(0)
+           and k_cache.size(3) == q.size(3), "q [B, T, Hq, d] and caches [B, Hkv, max_len, d] expected")
+    B, T, Hq, d = q.shape
+    Hkv, max_len = k_cache.size(1), k_cache.size(2)
+    _check(d == 128, "head_dim must be 128")
+    _check(Hkv > 0 and Hq % Hkv == 0, "Hq must be a multiple of Hkv")
+    past = int(past)
+    _check(past >= 0 and past + T <= max_len, "past + T must fit the cache")
+    out = torch.empty((B, T, Hq * d), dtype=torch.float16, device=q.device)
+    if B and T:
+        _run("flh_prefill_attention_f16", q.device, q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(), B, T,
+             Hq, Hkv, d, past, max_len, float(scale if scale is not None else d ** -0.5), _stream(q))
+    return out
+
+
 def decode_attention(q, k_cache, v_cache, kv_len, scale=None, workspace=None):
     """One new token per sequence against the first `kv_len` slots of a preallocated cache: q [B, Hq, d] fp16,
     k_cache / v_cache [B, Hkv, max_len, d] fp16 -> [B, Hq, d] fp16 = softmax(q K^T * scale) V with float32 scores,

@@ -12,7 +12,7 @@ import sys
 
 HERE = pathlib.Path(__file__).resolve().parent
 OUT = HERE.parent / "libflh_hip.so"
-SOURCES = ["capi.hip", "reference_abi.hip", "gemm_i4.hip", "gemm_i4_decode.hip", "gemm_f6.hip", "fwht_quant.hip", "fwht_mfma.hip", "rope_cache.hip", "decode_attention.hip"]
+SOURCES = ["capi.hip", "reference_abi.hip", "gemm_i4.hip", "gemm_i4_decode.hip", "gemm_f6.hip", "fwht_quant.hip", "fwht_mfma.hip", "rope_cache.hip", "decode_attention.hip", "prefill_attention.hip"]
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",

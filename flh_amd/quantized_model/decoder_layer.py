@@ -312,6 +312,8 @@ class W4A4DecoderLayer(torch.nn.Module):
             ks, vs = kv_cache.rope_and_update(qs, ks.view(b, t, self.num_kv_heads, self.head_dim),
                                               vs.view(b, t, self.num_kv_heads, self.head_dim), cos, sin, positions)
             cache = kv_cache
+            if self._own_prefill_attention(t):
+                out = _ops().prefill_attention(qs, *kv_cache.tensors(), kv_cache.owner.kv_len - t)
             qs = qs.transpose(1, 2)
         elif (self.fused and x.is_cuda and self.head_dim % 16 == 0 and cos.dtype == torch.float16
               and cos.shape == (t, self.head_dim)):
@@ -328,6 +330,8 @@ class W4A4DecoderLayer(torch.nn.Module):
             _ops().rope_kv_cache_(qs, ks.view(b, t, self.num_kv_heads, self.head_dim),
                                   vs.view(b, t, self.num_kv_heads, self.head_dim), cos.contiguous(), sin.contiguous(),
                                   slots, keys, values)
+            if self._own_prefill_attention(t):
+                out = _ops().prefill_attention(qs, keys, values, past)
             qs = qs.transpose(1, 2)
             ks, vs = keys, values
             cache = (ks, vs)
@@ -369,6 +373,11 @@ class W4A4DecoderLayer(torch.nn.Module):
         self._tap("o_proj", y)
         return x, y, cache
 
+    def _own_prefill_attention(self, t):
+        """Whether a block of t > 1 new tokens takes this library's causal-attention kernel (heads of 128 channels) instead
+        of torch's fused attention."""
+        return self.fused and self.record is None and t > 1 and self.head_dim == 128
+
     def _qkv_rope_applies(self, rows, codes, scales, cos, kv_cache, positions):
         """Whether q / k / v take the launch whose epilogue applies the rotary embedding and writes the cache: the fused
         prefill path with heads of 128 channels, nibble codes that stay on the int8 kernel (not the 6-bit format, no layer
@@ -408,18 +417,11 @@ class W4A4DecoderLayer(torch.nn.Module):
         qs = _ops().gemm_i4_qkv_rope(codes.reshape(b * t, -1), scales.reshape(b * t, -1),
                                      [l.w_packed.view(l.out_features, l.in_features // 2) for l in layers],
                                      [l.w_scale.view(l.out_features, -1) for l in layers], cos.contiguous(),
-                                     sin.contiguous(), slots, keys, values, b, group).transpose(1, 2)
+                                     sin.contiguous(), slots, keys, values, b, group)
         if static:
-            n = kv_cache.owner.kv_len
-            keys, values = keys[:, :, :n], values[:, :, :n]
-            past = n - t
-        gqa = self.num_heads != self.num_kv_heads
-        if past == 0:
-            out = torch.nn.functional.scaled_dot_product_attention(qs, keys, values, is_causal=t > 1, enable_gqa=gqa)
-        else:
-            mask = torch.ones(t, past + t, dtype=torch.bool, device=x.device).tril(diagonal=past)
-            out = torch.nn.functional.scaled_dot_product_attention(qs, keys, values, attn_mask=mask, enable_gqa=gqa)
-        out = out.transpose(1, 2).reshape(b, t, self.hidden_size).contiguous()
+            past = kv_cache.owner.kv_len - t
+        # causal attention of the new block over the cache slots 0 .. past + t - 1, this library's kernel (heads of 128)
+        out = _ops().prefill_attention(qs, keys, values, past)
         return self._output_projection(x, out, cache, fold_residual)
 
     def _residual_in_gemm(self, rows):

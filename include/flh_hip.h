@@ -326,6 +326,16 @@ int flh_rope_kv_cache_f16(flh_half* q, const flh_half* k, const flh_half* v, con
                           const int64_t* positions, flh_half* k_cache, flh_half* v_cache, uint32_t B, uint32_t T,
                           uint32_t Hq, uint32_t Hkv, uint32_t head_dim, uint32_t max_len, void* stream);
 
+/* Causal attention of a block of T new tokens per sequence over the cache (prefill): query t sees the slots 0 .. past + t of
+ * its sequence's keys / values (the block's own keys / values sit in slots past .. past + T - 1, where flh_rope_kv_cache_f16
+ * or flh_gemm_i4_qkv_rope_o16 put them).  Stands where the reference calls flash-attn on the rotated projections
+ * (flh/quantized_model/modeling_llama.py:426-460).  q [B, T, Hq, 128] fp16 (token-major, as those launches write it),
+ * k_cache / v_cache [B, Hkv, max_len, 128], out [B, T, Hq * 128] fp16; head_dim must be 128, Hq a multiple of Hkv;
+ * softmax(scale * q . k) in float32, probabilities rounded to fp16 for the second product, float32 accumulation. */
+int flh_prefill_attention_f16(const flh_half* q, const flh_half* k_cache, const flh_half* v_cache, flh_half* out, uint32_t B,
+                              uint32_t T, uint32_t Hq, uint32_t Hkv, uint32_t head_dim, uint32_t past, uint32_t max_len,
+                              float scale, void* stream);
+
 /* Attention of ONE new token per sequence over the cache that flh_rope_kv_cache_f16 fills (the decode step), grouped
  * queries included:  out[b, h] = softmax(q[b, h] . K[b, h / rep]^T * scale) V[b, h / rep]  over cache slots [0, kv_len),
  * rep = Hq / Hkv in {1, 2, 4, 8}, head_dim 64 or 128; scores, probabilities and sums in float32, fp16 in and out.

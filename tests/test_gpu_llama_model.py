@@ -288,11 +288,13 @@ def test_llama2_layer_8x512_against_the_oracle():
     with torch.no_grad():
         y, (k, v) = layer(x, cos, sin)
     assert torch.equal(k, k_rec) and torch.equal(v, v_rec)
-    # the production run computes silu(gate) * up inside the gate / up launch (device exponential) where the recorded
-    # run used torch's kernels: the same values but for a last fp16 bit here and there
+    # the production run computes silu(gate) * up inside the gate / up launch (device exponential) and attention with the
+    # library's own kernel where the recorded run used torch's kernels: the same values but for a last fp16 bit here and
+    # there, which the two int4 quantisers behind them turn into a few per cent of the layer's update (far below the
+    # int4 noise itself, which the stage checks below bound against the oracle)
     rel = ((y.float() - y_rec.float()).norm() / (y_rec.float() - x.float()).norm()).item()
-    print(f"  fused gate/up launch vs module sequence: relative difference of the layer's update {rel:.2e}", flush=True)
-    assert rel < 2e-2
+    print(f"  production launches vs module sequence: relative difference of the layer's update {rel:.2e}", flush=True)
+    assert rel < 5e-2
     rec = {kk: host(vv).reshape(-1, vv.shape[-1]) for kk, vv in rec.items()}
     sample = np.sort(np.random.default_rng(4).choice(b * t, 192, replace=False))
     out, report = check_layer_stages(rec, w, host(x).reshape(b * t, hidden), host(cos), host(sin), b, t, None,

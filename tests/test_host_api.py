@@ -74,6 +74,10 @@ def test_argument_errors_come_back_before_any_launch():
         ("flh_decode_attention_f16", (ok, ok, ok, ok, 1, 32, 8, 128, 2048, 2048, 1.0, ok, 16, st), b"workspace"),
         ("flh_decode_attention_f16_static", (ok, ok, ok, ok, 4096, 32, 8, 128, 8192, 8192, 1.0, st), b"static array"),
         ("flh_gemm_set_tuning", (100, 0), b"tile must be"),
+        ("flh_prefill_attention_f16", (ok, ok, ok, ok, 1, 16, 8, 2, 64, 0, 64, 0.1, st), b"head_dim (64) must be 128"),
+        ("flh_prefill_attention_f16", (ok, ok, ok, ok, 1, 16, 8, 3, 128, 0, 64, 0.1, st), b"do not divide"),
+        ("flh_prefill_attention_f16", (ok, ok, ok, ok, 1, 16, 8, 2, 128, 60, 64, 0.1, st), b"exceeds the cache length"),
+        ("flh_prefill_attention_f16", (ok, odd, ok, ok, 1, 16, 8, 2, 128, 0, 64, 0.1, st), b"16-byte aligned"),
         ("flh_gemm_i4_add_o16", (ok, ok, ok, ok, odd, ok, 16, 128, 128, 1, 1, 128, st), b"residual must be 16-byte aligned"),
         ("flh_gemm_i4_add_o16", (ok, ok, ok, ok, None, ok, 16, 128, 128, 1, 1, 128, st), b"null pointer"),
         ("flh_gemm_f6_add_o16", (ok, ok, ok, ok, ok, ok, 16, 128, 256, 3, 2, st), b"scale columns"),
