@@ -52,8 +52,12 @@ __global__ __launch_bounds__(256, 2) void prefill_attention_kernel(const __half*
   // blocks (late queries) come first
   const int n_blocks = (T + kQueriesPerBlock - 1) / kQueriesPerBlock;
   const unsigned L = xcd_contiguous(blockIdx.x, gridDim.x);
-  const int qb = n_blocks - 1 - (int)(L % n_blocks);
   const int head = (int)((L / n_blocks) % Hq), b = (int)(L / ((unsigned)n_blocks * Hq));
+  // a die's 32 compute units take its workgroups in order, two each: every other row of 32 workgroups walks its heads'
+  // blocks in the opposite direction, so that a compute unit's two residents are a long and a short block
+  // (heads of 32 blocks or more fill whole rows: they keep the long blocks first)
+  const bool ascending = n_blocks < 32 && (((L / n_blocks) / (32 / n_blocks)) & 1);
+  const int qb = ascending ? (int)(L % n_blocks) : n_blocks - 1 - (int)(L % n_blocks);
   const int hkv = head / (Hq / Hkv);
   const int q_first = qb * kQueriesPerBlock + wave * 32;
   const int my_q = min(q_first + n, T - 1);            // rows past the end repeat the last query; never stored
