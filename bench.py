@@ -676,12 +676,28 @@ def main():
             layer_fig[f"token_configuration,prefill_8x512,{label}_us"] = round(wall_us(lambda: layer(xs8, cos8, sin8), reps=20), 1)
             del layer
     del lw, xs, xs8
+    # the causal attention kernel of the prefill path alone, beside torch's fused attention on the same tensors
+    attn_fig = {}
+    for (ab, at, ahq, ahkv) in ((8, 512, 32, 32), (1, 2048, 32, 32), (1, 2048, 32, 8)):
+        aq = torch.randn(ab, at, ahq, 128, generator=gen).half().to(dev)
+        ak = torch.randn(ab, ahkv, at, 128, generator=gen).half().to(dev)
+        av = torch.randn(ab, ahkv, at, 128, generator=gen).half().to(dev)
+        aqt = aq.transpose(1, 2)
+        us_own = timed([lambda: ops.prefill_attention(aq, ak, av, 0)] * 20)
+        us_torch = timed([lambda: torch.nn.functional.scaled_dot_product_attention(aqt, ak, av, is_causal=True,
+                                                                                   enable_gqa=ahq != ahkv)] * 20)
+        flops = 4 * ab * ahq * at * at * 128 / 2
+        attn_fig[f"{ab}x{at}_tokens,{ahq}/{ahkv}_heads"] = {"us": round(us_own, 1), "TFLOP/s": round(flops / us_own / 1e6, 1),
+                                                         "torch_fused_attention_us": round(us_torch, 1)}
+        del aq, ak, av, aqt
+    layer_fig["prefill_attention_kernel"] = attn_fig
 
     # The Llama-3-8B decode step (32 layers, batch x 1 token, attention over 2048 cached positions, grouped queries 32 / 8,
     # intermediate 14336 with the 28 x 512 online rotation, group-of-128 weight scales, fp16 head of 128 256 rows), random
-    # weights, captured into one graph and replayed.  Only the int4 linears and their quantisers are this library's
-    # kernels; embedding, RoPE, cache write, attention, residual adds, SiLU, the final norm and the head are stock torch
-    # ops and are reported separately (whole step minus the same step's linears-only graph).  Lower bound of the step:
+    # weights, captured into one graph and replayed.  The int4 linears and their quantisers (with the norms, residual
+    # additions and SiLU inside), the rotary embedding, the cache write and attention are this library's kernels; the
+    # embedding, the final norm and the fp16 head are torch's.  "everything else" = whole step minus the same step's
+    # linears-and-quantisers graph.  Lower bound of the step:
     # all int4 weights and scales + the fp16 head + the cached keys / values once over HBM.
     from flh_amd.quantized_model import LlamaShape, W4A4LlamaModel
     decode_model = {}
