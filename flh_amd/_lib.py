@@ -30,6 +30,9 @@ _SIG = {
                                             _c.c_int, _c.c_int, _PTR]),
     "flh_prefill_attention_f16": (_c.c_int, [_PTR, _PTR, _PTR, _PTR, _c.c_uint32, _c.c_uint32, _c.c_uint32, _c.c_uint32,
                                              _c.c_uint32, _c.c_uint32, _c.c_uint32, _c.c_float, _PTR]),
+    "flh_gemm_f6_qkv_rope_o16": (_c.c_int, [_PTR, _PTR, _PTR, _PTR, _PTR, _PTR, _PTR, _PTR, _PTR, _PTR, _c.c_uint32,
+                                            _c.c_uint32, _c.c_uint32, _c.c_uint32, _c.c_uint32, _c.c_size_t, _c.c_int,
+                                            _c.c_int, _PTR]),
     "flh_gemm_i4_swiglu_o16": (_c.c_int, [_PTR, _PTR, _PTR, _PTR, _PTR, _PTR, _PTR, _c.c_size_t, _c.c_size_t, _c.c_size_t,
                                           _c.c_int, _c.c_int, _c.c_int, _PTR]),
     "flh_gemm_f6_swiglu_o16": (_c.c_int, [_PTR, _PTR, _PTR, _PTR, _PTR, _PTR, _PTR, _c.c_size_t, _c.c_size_t, _c.c_size_t,

@@ -432,6 +432,32 @@ def gemm_f6_dequant_add(A6, B6, A_scale, B_scale, residual, out=None):
     return D
 
 
+def gemm_f6_qkv_rope(A6, A_scale, B6s, B_scales, cos, sin, positions, k_cache, v_cache, batch):
+    """gemm_i4_qkv_rope on operands encoded by encode_f6 (or written by rotate_and_quantize_f6): scales all one column, or
+    weight scales [N, K/128] with A_scale [M, 1] or [M, K/128].  Same bits."""
+    import ctypes
+    _check(len(B6s) == 3 and len(B_scales) == 3, "three weight matrices (q, k, v), one scale tensor each")
+    M = K = None
+    for B6, S in zip(B6s, B_scales):
+        m, n, k = _check_f6(A6, B6)
+        M, K = m, k
+        _check(S.is_cuda and S.dtype == torch.float16 and S.is_contiguous() and S.dim() == 2 and S.size(0) == n
+               and S.size(1) == B_scales[0].size(1) and S.device == A6.device, "B_scale shapes")
+    ng = K // 128
+    _check(A_scale.is_cuda and A_scale.dtype == torch.float16 and A_scale.is_contiguous() and A_scale.dim() == 2
+           and A_scale.size(0) == M and A_scale.device == A6.device, "A_scale must be a contiguous float16 CUDA tensor [M, .]")
+    _check((A_scale.size(1), B_scales[0].size(1)) in ((1, 1), (1, ng), (ng, ng)),
+           "scale columns must be (1, 1), (1, K/128) or (K/128, K/128)")
+    T, Hq, Hkv, max_len = _check_rope_cache(M, batch, B6s, cos, sin, positions, k_cache, v_cache, A6.device)
+    q_out = torch.empty((batch, T, Hq, 128), dtype=torch.float16, device=A6.device)
+    if M:
+        ptrs = lambda ts: (ctypes.c_void_p * 3)(*[t.data_ptr() for t in ts])
+        _run("flh_gemm_f6_qkv_rope_o16", A6.device, A6.data_ptr(), A_scale.data_ptr(), ptrs(B6s), ptrs(B_scales),
+             cos.data_ptr(), sin.data_ptr(), positions.data_ptr(), q_out.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
+             batch, T, Hq, Hkv, max_len, K, A_scale.size(1), B_scales[0].size(1), _stream(A6))
+    return q_out
+
+
 def gemm_f6_swiglu(A6, B6_gate, B6_up, A_scale, gate_scale, up_scale):
     """gemm_i4_swiglu on operands encoded by encode_f6 (or written by rotate_and_quantize_f6): fp16(fp16(silu(gate)) * up)
     in one launch, gate / up = gemm_f6_dequant_o16[_gs](A6, B6_gate / B6_up, ...); scales all one column, or weight scales

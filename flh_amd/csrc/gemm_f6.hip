@@ -48,7 +48,10 @@ typedef int v8i __attribute__((ext_vector_type(8)));
 // workgroup -- the tile's BN weight rows are BN / 2 rows of the gate matrix and the same BN / 2 rows of the up matrix, the
 // two wave columns -- rounds both to fp16 as their own launches would store them, and stores only
 // fp16(fp16(silu(gate)) * up): [M, N] with N the width of ONE of the matrices.
-template <int BM, int BN, int WM, int WN, int STAGES, int EPI, bool SWIGLU = false>
+//
+// ROPE (as in the int8 kernel): a q / k / v launch with heads of 128 channels = one tile column each, whose epilogue
+// applies the rotary embedding to the query and key heads and writes keys and values into their cache slots.
+template <int BM, int BN, int WM, int WN, int STAGES, int EPI, bool SWIGLU = false, bool ROPE = false>
 __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN), ((BM / WM) * (BN / WN) == 4 && WM * WN <= 64 * 64) ? 2 : 1)
 void gemm_f6_kernel(const GemmArgs p) {
   constexpr int TM = WM / 32, TN = WN / 32;
@@ -62,6 +65,7 @@ void gemm_f6_kernel(const GemmArgs p) {
   constexpr int EPI_PITCH = WN * 2 + kEpiPadF6;
   static_assert((WAVES == 4 || WAVES == 8) && BM % 64 == 0 && BN % 64 == 0, "tile shape");
   static_assert(!SWIGLU || (EPI != kInt32 && WAVES_N == 2), "gate | up halves are the two wave columns");
+  static_assert(!ROPE || (EPI != kInt32 && BN == 128 && WN == 64 && !SWIGLU), "a tile column is one head of 128");
   constexpr int BNC = SWIGLU ? BN / 2 : BN;           // output channels per tile
   static_assert((BM + BN) * 6 % 64 == 0 && (BM * 6) % 64 == 0, "whole load instructions, none straddling A | B");
   static_assert(STAGES >= 3, "ring depth");
@@ -91,7 +95,7 @@ void gemm_f6_kernel(const GemmArgs p) {
   const uint8_t* wB = p.B;
   const __half* wBs = p.Bs;
   void* wD = p.D;
-  int wN = p.N, seg_tile = tile_n;
+  int wN = p.N, seg_tile = tile_n, seg = 0;
   for (int s = 1; s < p.n_seg; ++s)
     if (tile_n >= p.seg_tile0[s]) {
       wB = p.seg_B[s];
@@ -99,6 +103,7 @@ void gemm_f6_kernel(const GemmArgs p) {
       wD = p.seg_D[s];
       wN = p.seg_N[s];
       seg_tile = tile_n - p.seg_tile0[s];
+      seg = s;
     }
   const int m0 = tile_m * BM, n0 = seg_tile * BNC;
 
@@ -405,6 +410,75 @@ void gemm_f6_kernel(const GemmArgs p) {
       }
       return;
     }
+    if constexpr (ROPE) {
+      // the tile's 128 columns are one head: its first 64 channels sit in the left wave column's staging tile, the other
+      // 64 in the right one's; each of the two waves finishes half of the band's rows, both halves of every row.  The
+      // table entries and cache slots of all rows are requested before the barrier.
+      constexpr int NIT = WM / (2 * RPI);
+      const int wcol = wave % WAVES_N;
+      const int head = seg_tile;
+      h8 c1[NIT], c2[NIT], s1[NIT], s2[NIT];
+      long long slot[NIT];
+      int bi[NIT];
+      {
+        const int m_first = m0 + wm + wcol * (WM / 2) + crow;
+        int b = m_first / p.rope_T, tt = m_first - b * p.rope_T;
+#pragma unroll
+        for (int it = 0; it < NIT; ++it) {
+          const int m = m_first + it * RPI;
+          const int tc = m < p.M ? tt : 0;               // rows past the end: any valid table row, nothing is stored
+          bi[it] = b;
+          slot[it] = seg == 0 ? 0 : p.rope_pos[tc];
+          if (seg < 2) {
+            const __half* ct = p.rope_cos + (size_t)tc * 128 + cchunk * 8;
+            const __half* st = p.rope_sin + (size_t)tc * 128 + cchunk * 8;
+            c1[it] = *(const h8*)ct, c2[it] = *(const h8*)(ct + 64), s1[it] = *(const h8*)st, s2[it] = *(const h8*)(st + 64);
+          }
+          tt += RPI;
+          while (tt >= p.rope_T) tt -= p.rope_T, ++b;
+        }
+      }
+      __syncthreads();
+      const uint8_t* lo_t = lds + (wave - wcol) * (WM * EPI_PITCH);
+      const uint8_t* hi_t = lo_t + WM * EPI_PITCH;
+#pragma unroll
+      for (int it = 0; it < NIT; ++it) {
+        const int row = wcol * (WM / 2) + it * RPI + crow;
+        const int m = m0 + wm + row;
+        h8 x1 = *(const h8*)(lo_t + row * EPI_PITCH + cchunk * 16);
+        h8 x2 = *(const h8*)(hi_t + row * EPI_PITCH + cchunk * 16);
+        if (m < p.M) {
+          bool in_range = true;
+          __half* dst;
+          if (seg == 0) {
+            dst = (__half*)wD + (size_t)m * wN + head * 128;
+          } else {
+            in_range = slot[it] >= 0 && slot[it] < (long long)p.rope_max_len;
+            dst = (__half*)wD +
+                  (((size_t)bi[it] * p.rope_hkv + head) * p.rope_max_len + (size_t)(in_range ? slot[it] : 0)) * 128;
+          }
+          if (seg < 2) {                                 // queries and keys: fp16(fp16(x cos) + fp16(rotate_half(x) sin))
+            h8 y1, y2;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+              const _Float16 a1 = (_Float16)round_here((float)x1[e] * (float)c1[it][e]);
+              const _Float16 r1 = (_Float16)round_here(-1.f * (float)x2[e] * (float)s1[it][e]);
+              y1[e] = (_Float16)round_here((float)a1 + (float)r1);
+              const _Float16 a2 = (_Float16)round_here((float)x2[e] * (float)c2[it][e]);
+              const _Float16 r2 = (_Float16)round_here(1.f * (float)x1[e] * (float)s2[it][e]);
+              y2[e] = (_Float16)round_here((float)a2 + (float)r2);
+            }
+            x1 = y1;
+            x2 = y2;
+          }
+          if (in_range) {
+            *(h8*)(dst + cchunk * 8) = x1;
+            *(h8*)(dst + 64 + cchunk * 8) = x2;
+          }
+        }
+      }
+      return;
+    }
     // ... and write it out as whole row segments (the tile is private to the wave: no barrier)
 #pragma unroll
     for (int it = 0; it < WM / RPI; ++it) {
@@ -427,7 +501,7 @@ void gemm_f6_kernel(const GemmArgs p) {
   }
 }
 
-template <int BM, int BN, int WM, int WN, int STAGES, int EPI, bool SWIGLU = false>
+template <int BM, int BN, int WM, int WN, int STAGES, int EPI, bool SWIGLU = false, bool ROPE = false>
 int launch_f6(GemmArgs a, hipStream_t stream) {
   constexpr int BNC = SWIGLU ? BN / 2 : BN;           // output channels per tile
   a.tiles_m = (a.M + BM - 1) / BM;
@@ -439,7 +513,7 @@ int launch_f6(GemmArgs a, hipStream_t stream) {
   a.group_m = a.tiles_m < 4 ? a.tiles_m : 4;
   const size_t smem = (size_t)STAGES * (BM + BN) * kBlockBytes +
                       (EPI == kRowScale ? (BM + BN) * 2 : (EPI == kGroupScale || EPI == kTokenGroup) ? (BM + BN) * 32 : 0);
-  auto kern = gemm_f6_kernel<BM, BN, WM, WN, STAGES, EPI, SWIGLU>;
+  auto kern = gemm_f6_kernel<BM, BN, WM, WN, STAGES, EPI, SWIGLU, ROPE>;
   static std::atomic<bool> attr_set{false};   // set-up is idempotent: a race only repeats it  // per instantiation
   if (!attr_set.load(std::memory_order_acquire)) {
     if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess)
@@ -605,6 +679,49 @@ extern "C" int flh_gemm_f6_swiglu_o16(const uint8_t* A6, const uint8_t* B6_gate,
   if (!grouped) return launch_f6_swiglu<kRowScale>(g, (hipStream_t)stream);
   if (a_cols == 1) return launch_f6_swiglu<kTokenGroup>(g, (hipStream_t)stream);
   return launch_f6_swiglu<kGroupScale>(g, (hipStream_t)stream);
+}
+
+extern "C" int flh_gemm_f6_qkv_rope_o16(const uint8_t* A6, const flh_half* a_scale, const uint8_t* const* B6,
+                                        const flh_half* const* b_scale, const flh_half* cos, const flh_half* sin,
+                                        const int64_t* positions, flh_half* q_out, flh_half* k_cache, flh_half* v_cache,
+                                        uint32_t batch, uint32_t T, uint32_t Hq, uint32_t Hkv, uint32_t max_len, size_t K,
+                                        int a_cols, int b_cols, void* stream) {
+  if (!B6 || !b_scale) return fail(FLH_EINVAL, "gemm_f6 (q/k/v + rotary): null array");
+  if (Hq == 0 || Hkv == 0 || max_len == 0)
+    return fail(FLH_EINVAL, "gemm_f6 (q/k/v + rotary): heads and cache length must be positive");
+  const size_t M = (size_t)batch * T;
+  const size_t N[3] = {(size_t)Hq * 128, (size_t)Hkv * 128, (size_t)Hkv * 128};
+  flh_half* const D[3] = {q_out, k_cache, v_cache};
+  for (int s = 0; s < 3; ++s) {
+    if (int e = check_f6(A6, B6[s], D[s], M, N[s], K)) return e;
+    if (!b_scale[s]) return fail(FLH_EINVAL, "gemm_f6: null scale pointer");
+  }
+  if (M == 0) return FLH_OK;
+  if (!a_scale || !cos || !sin || !positions) return fail(FLH_EINVAL, "gemm_f6 (q/k/v + rotary): null pointer");
+  if (misaligned16(cos, sin)) return fail(FLH_EINVAL, "gemm_f6 (q/k/v + rotary): cos and sin must be 16-byte aligned");
+  if ((uint64_t)batch * Hkv * max_len > (1ull << 40) / 128) return fail(FLH_EINVAL, "gemm_f6 (q/k/v + rotary): cache too large");
+  const int ng = (int)(K / 128);
+  const bool rows_only = a_cols == 1 && b_cols == 1;
+  if (!rows_only && (b_cols != ng || (a_cols != 1 && a_cols != ng)))
+    return fail(FLH_EINVAL, "gemm_f6: scale columns (%d, %d) must be (1, 1) or (1 or K/128, K/128) with K/128 = %d", a_cols, b_cols, ng);
+  GemmArgs g{A6, B6[0], (const __half*)a_scale, (const __half*)b_scale[0], q_out, (int)M, (int)N[0], (int)K, a_cols, b_cols, 0, 0, 0};
+  g.n_seg = 3;
+  for (int s = 1; s < 3; ++s) {
+    g.seg_B[s] = B6[s];
+    g.seg_Bs[s] = (const __half*)b_scale[s];
+    g.seg_D[s] = D[s];
+    g.seg_N[s] = (int)N[s];
+  }
+  g.rope_cos = (const __half*)cos;
+  g.rope_sin = (const __half*)sin;
+  g.rope_pos = (const long long*)positions;
+  g.rope_T = (int)T;
+  g.rope_max_len = (int)max_len;
+  g.rope_hkv = (int)Hkv;
+  // 128 x 128 tiles (a tile column = one head)
+  if (rows_only) return launch_f6<128, 128, 64, 64, 3, kRowScale, false, true>(g, (hipStream_t)stream);
+  if (a_cols == 1) return launch_f6<128, 128, 64, 64, 3, kTokenGroup, false, true>(g, (hipStream_t)stream);
+  return launch_f6<128, 128, 64, 64, 3, kGroupScale, false, true>(g, (hipStream_t)stream);
 }
 
 extern "C" int flh_gemm_f6_o16_multi(const uint8_t* A6, const flh_half* a_scale, int count, const uint8_t* const* B6,

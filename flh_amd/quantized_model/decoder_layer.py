@@ -288,8 +288,9 @@ class W4A4DecoderLayer(torch.nn.Module):
         else:
             x, s, z, q = self._residual_norm_quant("attn_in", self.input_layernorm, "input_layernorm",
                                                    self.attn_quantizer1, x, add, (self.q_proj, self.k_proj, self.v_proj))
-            if self._qkv_rope_applies(b * t, q, s, cos, kv_cache, positions):
-                return self._attention_after_fused_qkv(x, q, s, cos, sin, kv_cache, positions, fold_residual)
+            mode = self._qkv_rope_applies(b * t, q, s, cos, kv_cache, positions)
+            if mode:
+                return self._attention_after_fused_qkv(x, q, s, cos, sin, kv_cache, positions, fold_residual, mode)
             qs, ks, vs = self._project([self.q_proj, self.k_proj, self.v_proj], q, s, z)
         self._tap("q_proj", qs), self._tap("k_proj", ks), self._tap("v_proj", vs)
         static = isinstance(kv_cache, StaticKVCache._Layer)
@@ -379,22 +380,25 @@ class W4A4DecoderLayer(torch.nn.Module):
         return self.fused and self.record is None and t > 1 and self.head_dim == 128
 
     def _qkv_rope_applies(self, rows, codes, scales, cos, kv_cache, positions):
-        """Whether q / k / v take the launch whose epilogue applies the rotary embedding and writes the cache: the fused
-        prefill path with heads of 128 channels, nibble codes that stay on the int8 kernel (not the 6-bit format, no layer
-        that would re-encode them) and fp16 tables."""
+        """Whether q / k / v take the launch whose epilogue applies the rotary embedding and writes the cache -- the fused
+        prefill path with heads of 128 channels and fp16 tables -- and on which matrix instruction: "i4" (nibble codes on
+        the int8 kernel), "f6" (codes in the 6-bit format, or layers that would re-encode them) or None."""
         static = isinstance(kv_cache, StaticKVCache._Layer)
+        if not (self.fused and self.record is None and rows > 64 and rows > codes.size(0) and self.head_dim == 128
+                and codes.is_cuda and self._online_qkv_applies() and cos.dtype == torch.float16
+                and tuple(cos.shape) == (rows // codes.size(0), 128) and (positions is not None if static else True)):
+            return None
+        if codes.size(-1) * 4 == self.hidden_size * 3:
+            return "f6"
+        if codes.size(-1) * 2 != self.hidden_size:
+            return None
         layers = (self.q_proj, self.k_proj, self.v_proj)
         group = self.q_proj.weight_group_size if self.q_proj.weight_group_size > 0 else (self.q_proj.in_group_size or 128)
-        if codes.size(-1) * 2 == self.hidden_size and all(
-                l._six_bit_applies(codes.reshape(rows, -1), scales.reshape(rows, -1), l.w_scale.view(l.out_features, -1), group)
-                for l in layers):
-            return False
-        return (self.fused and self.record is None and rows > 64 and rows > codes.size(0) and self.head_dim == 128 and codes.is_cuda
-                and codes.size(-1) * 2 == self.hidden_size and self._online_qkv_applies()
-                and cos.dtype == torch.float16 and tuple(cos.shape) == (rows // codes.size(0), 128)
-                and (positions is not None if static else True))
+        six = all(l._six_bit_applies(codes.reshape(rows, -1), scales.reshape(rows, -1), l.w_scale.view(l.out_features, -1), group)
+                  for l in layers)
+        return "f6" if six else "i4"
 
-    def _attention_after_fused_qkv(self, x, codes, scales, cos, sin, kv_cache, positions, fold_residual):
+    def _attention_after_fused_qkv(self, x, codes, scales, cos, sin, kv_cache, positions, fold_residual, mode):
         """The prefill attention block from the quantised input on: q / k / v, rotary embedding and cache write in one
         launch (the bits of the separate launches), torch's fused attention, then the output projection."""
         b, t, _ = x.shape
@@ -414,10 +418,15 @@ class W4A4DecoderLayer(torch.nn.Module):
             slots = torch.arange(past, past + t, device=x.device)
             cache = (keys, values)
         group = self.q_proj.weight_group_size if self.q_proj.weight_group_size > 0 else (self.q_proj.in_group_size or 128)
-        qs = _ops().gemm_i4_qkv_rope(codes.reshape(b * t, -1), scales.reshape(b * t, -1),
-                                     [l.w_packed.view(l.out_features, l.in_features // 2) for l in layers],
-                                     [l.w_scale.view(l.out_features, -1) for l in layers], cos.contiguous(),
-                                     sin.contiguous(), slots, keys, values, b, group)
+        w_scales = [l.w_scale.view(l.out_features, -1) for l in layers]
+        rows, a_rows = codes.reshape(b * t, -1), scales.reshape(b * t, -1)
+        if mode == "f6":
+            a6 = rows.contiguous() if rows.size(1) * 4 == self.hidden_size * 3 else _ops().encode_f6(rows.contiguous())
+            qs = _ops().gemm_f6_qkv_rope(a6, a_rows.contiguous(), [l._six_bit_weights() for l in layers], w_scales,
+                                         cos.contiguous(), sin.contiguous(), slots, keys, values, b)
+        else:
+            qs = _ops().gemm_i4_qkv_rope(rows, a_rows, [l.w_packed.view(l.out_features, l.in_features // 2) for l in layers],
+                                         w_scales, cos.contiguous(), sin.contiguous(), slots, keys, values, b, group)
         if static:
             past = kv_cache.owner.kv_len - t
         # causal attention of the new block over the cache slots 0 .. past + t - 1, this library's kernel (heads of 128)

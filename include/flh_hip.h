@@ -220,6 +220,13 @@ int flh_gemm_f6_add_o16(const uint8_t* A6, const uint8_t* B6, const flh_half* a_
                         const flh_half* residual, flh_half* D, size_t M, size_t N, size_t K, int a_cols, int b_cols,
                         void* stream);
 
+/* flh_gemm_i4_qkv_rope_o16 on 6-bit operands (a_cols = b_cols = 1, or groups of 128 as in flh_gemm_f6_o16_gs); same bits. */
+int flh_gemm_f6_qkv_rope_o16(const uint8_t* A6, const flh_half* a_scale, const uint8_t* const* B6,
+                             const flh_half* const* b_scale, const flh_half* cos, const flh_half* sin,
+                             const int64_t* positions, flh_half* q_out, flh_half* k_cache, flh_half* v_cache,
+                             uint32_t batch, uint32_t T, uint32_t Hq, uint32_t Hkv, uint32_t max_len, size_t K,
+                             int a_cols, int b_cols, void* stream);
+
 /* flh_gemm_i4_swiglu_o16 on 6-bit operands: gate = A . Bg^T and up = A . Bu^T in one launch that stores only
  * D[m, n] = fp16(fp16(silu(gate)) * up), [M, N] with N the width of one of the two encoded weight matrices.  a_cols = b_cols
  * = 1: one scale per row / channel; b_cols = K / 128 with a_cols 1 or K / 128: groups of 128.  Same bits as

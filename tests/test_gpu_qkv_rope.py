@@ -111,6 +111,26 @@ def test_qkv_rope_gemm_equals_the_two_launches_at_llama_width(ops):
     assert torch.equal(q, q2) and torch.equal(kc, kc2) and torch.equal(vc, vc2)
 
 
+@pytest.mark.parametrize("batch,t,hq,hkv,k", [(1, 70, 4, 4, 256), (3, 50, 4, 2, 512), (2, 300, 8, 2, 384), (1, 5, 2, 1, 128)])
+@pytest.mark.parametrize("scales", ["row", "token_group", "group_group"])
+def test_qkv_rope_gemm_on_the_six_bit_instruction(ops, batch, t, hq, hkv, k, scales):
+    """flh_gemm_f6_qkv_rope_o16: the same queries and cache bytes as the int8 launch (itself checked against the oracle)."""
+    from flh_amd.quantized_model import rotary_tables
+    a_cols, b_cols = {"row": (1, 1), "token_group": (1, 2), "group_group": (2, 2)}[scales]
+    print(f"case qkv rope f6 batch={batch} t={t} hq={hq} hkv={hkv} k={k} {scales}", flush=True)
+    ap, sa, ws, ss = case(batch, t, hq, hkv, k, batch + t + k + 7, a_cols, b_cols)
+    A, S, W, WS = dev(ap), dev(sa), [dev(w) for w in ws], [dev(s) for s in ss]
+    max_len = t + 11
+    pos = torch.randperm(max_len, device="cuda", generator=torch.Generator(device="cuda").manual_seed(3))[:t].contiguous()
+    cos, sin = rotary_tables(pos, 128, 10000.0)
+    kc = torch.full((batch, hkv, max_len, 128), 7.0, dtype=torch.float16, device="cuda")
+    vc = torch.full_like(kc, -3.0)
+    kc6, vc6 = kc.clone(), vc.clone()
+    q = ops.gemm_i4_qkv_rope(A, S, W, WS, cos, sin, pos, kc, vc, batch)
+    q6 = ops.gemm_f6_qkv_rope(ops.encode_f6(A), S, [ops.encode_f6(w) for w in W], WS, cos, sin, pos, kc6, vc6, batch)
+    assert torch.equal(q, q6) and torch.equal(kc, kc6) and torch.equal(vc, vc6)
+
+
 def test_qkv_rope_gemm_argument_checks(ops):
     ap, sa, ws, ss = case(1, 70, 4, 4, 256, 1, 1, 1)
     pos = torch.arange(70, device="cuda")

@@ -95,6 +95,12 @@ def test_argument_errors_come_back_before_any_launch():
     for kw, message in (({"k": 192}, b"multiple of 128"), ({"hkv": 0}, b"must be positive"), ({"cos": odd}, b"16-byte aligned"),
                         ({"b_cols": 2, "group": 64}, b"groups of 128")):
         assert rope(**kw) == -1 and message in lib.flh_last_error(), (kw, lib.flh_last_error())
+    rope6 = lambda **kw: lib.flh_gemm_f6_qkv_rope_o16(
+        ok, ok, three, three, kw.get("cos", ok), ok, ok, ok, ok, ok, 2, 40, 4, kw.get("hkv", 2), 64, kw.get("k", 256),
+        kw.get("a_cols", 1), kw.get("b_cols", 1), st)
+    for kw, message in (({"k": 192}, b"multiple of 128"), ({"hkv": 0}, b"must be positive"), ({"cos": odd}, b"16-byte aligned"),
+                        ({"a_cols": 3, "b_cols": 2}, b"scale columns")):
+        assert rope6(**kw) == -1 and message in lib.flh_last_error(), (kw, lib.flh_last_error())
 
 
 def test_ops_fail_loudly_without_library(monkeypatch, tmp_path):
