@@ -674,6 +674,12 @@ def main():
         for label, fused_form in (("module_by_module", False), ("fused", True)):
             layer = W4A4DecoderLayer.from_float(lw, 32, 32, fused=fused_form, activation="token")
             layer_fig[f"token_configuration,prefill_8x512,{label}_us"] = round(wall_us(lambda: layer(xs8, cos8, sin8), reps=20), 1)
+            if fused_form:
+                # ... with the rows of 4096 channels rotated on the matrix cores (the headline's rotation mode; the
+                # default keeps the bit-exact float32 butterflies in the layer)
+                layer.fast_rotation = True
+                layer_fig["token_configuration,prefill_8x512,fused,matrix_core_rotation_us"] = round(
+                    wall_us(lambda: layer(xs8, cos8, sin8), reps=20), 1)
             del layer
     del lw, xs, xs8
     # the causal attention kernel of the prefill path alone, beside torch's fused attention on the same tensors

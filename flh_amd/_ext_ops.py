@@ -46,8 +46,8 @@ def rotate_and_quantize_i4(x, hadamard=True, had_group=0, scale_group=0, clip_ra
 
 
 def rmsnorm_rotate_and_quantize_i4(x, weight, eps, hadamard=True, clip_ratio=1.0, return_rotated=False):
-    return tuple(_ext.rmsnorm_rotate_and_quantize_i4_mode(x, weight, eps, FLH_HAD_F32 if hadamard else FLH_HAD_NONE,
-                                                          clip_ratio, return_rotated))
+    return tuple(_ext.rmsnorm_rotate_and_quantize_i4_mode(x, weight, eps, _ops._whole_row_mode(hadamard), clip_ratio,
+                                                          return_rotated))
 
 
 def __getattr__(name):        # ops the extension does not wrap (6-bit path, int32 output, tuning hook, ...)

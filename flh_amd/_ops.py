@@ -792,6 +792,13 @@ def rmsnorm_and_quantize_i4_gs(x, weight, eps, group_size, hadamard=False, *, sc
     return [q, s]
 
 
+def _whole_row_mode(hadamard):
+    """hadamard argument of the power-of-two whole-row ops -> mode of the C ABI: False / None, True = "exact" (float32
+    butterflies), "fast" (matrix cores where a kernel exists: K = 4096; else the butterflies)."""
+    _check(hadamard in (True, False, None, "exact", "fast"), "hadamard must be True / 'exact', 'fast' or False")
+    return {True: FLH_HAD_F32, "exact": FLH_HAD_F32, "fast": FLH_HAD_MFMA, False: FLH_HAD_NONE, None: FLH_HAD_NONE}[hadamard]
+
+
 def rmsnorm_rotate_and_quantize_i4(x, weight, eps, hadamard=True, clip_ratio=1.0, return_rotated=False):
     """RMSNorm (flh/nn/normalization.py:12-20) + whole-row rotation + per-token quantiser in one launch:
     x [M, K] fp16, K in {512, ..., 8192}, weight [K] fp16 or None -> (q [M, K/2] u8, scales [M, 1] fp16
@@ -810,7 +817,7 @@ def rmsnorm_rotate_and_quantize_i4(x, weight, eps, hadamard=True, clip_ratio=1.0
     if M:
         _run("flh_rmsnorm_rotate_quant_i4", x.device, x.data_ptr(), weight.data_ptr() if weight is not None else None,
              float(eps), q.data_ptr(), s.data_ptr(), y.data_ptr() if y is not None else None, M, K,
-             FLH_HAD_F32 if hadamard else FLH_HAD_NONE, float(clip_ratio), _stream(x))
+             _whole_row_mode(hadamard), float(clip_ratio), _stream(x))
     return (q, s, y) if return_rotated else (q, s)
 
 
@@ -833,7 +840,7 @@ def add_rmsnorm_rotate_and_quantize_i4(x, add, weight, eps, hadamard=True, clip_
     if M:
         _run("flh_add_rmsnorm_rotate_quant_i4", x.device, x.data_ptr(), add.data_ptr(), total.data_ptr(),
              weight.data_ptr() if weight is not None else None, float(eps), q.data_ptr(), s.data_ptr(), M, K,
-             FLH_HAD_F32 if hadamard else FLH_HAD_NONE, float(clip_ratio), _stream(x))
+             _whole_row_mode(hadamard), float(clip_ratio), _stream(x))
     return total, q, s
 
 
@@ -852,8 +859,8 @@ def rotate_and_quantize_f6(x, hadamard=True, clip_ratio=1.0, norm_weight=None, e
         _check(hadamard in (True, "fast") and eps is None and add is None, "K = 11008 / 14336: matrix-core rotation, no prologue")
         mode = FLH_HAD_MFMA
     else:
-        _check(hadamard in (True, False, None, "exact"), "power-of-two K: hadamard True / 'exact' / False")
-        mode = FLH_HAD_F32 if hadamard in (True, "exact") else FLH_HAD_NONE
+        _check(hadamard != "fast" or K == 4096, "power-of-two K: the matrix-core rotation ('fast') exists for K = 4096")
+        mode = _whole_row_mode(hadamard)
     _check(add is None or eps is not None, "the residual addition comes with the RMSNorm prologue (eps)")
     if add is not None:
         _check(add.is_cuda and add.dtype == torch.float16 and add.shape == x.shape and add.is_contiguous()

@@ -81,13 +81,30 @@ __device__ __forceinline__ v4i quantise_block(const unsigned (&y0)[8], const uns
 // (s = k-step, h = lane / 32).  Level-2 slot map: (jb, s, h, i) holds
 // j = 32 jb + 16 s + 8 (i / 4) + 4 h + i % 4, which is where registers 8 s .. 8 s + 7 of the
 // level-1 accumulator tile jb sit.  The level-2 constants carry the 1/64 normalisation.
-template <bool SPLIT>
+//
+// Prologues and output format of the float32-butterfly kernels, on this rotation:
+//   ADD   the row is x + add in fp16 (one rounding per value), stored to sum_out as well (the residual stream);
+//   RMS   RMSNorm in front of the rotation (flh/nn/normalization.py:12-20): float32 sum of squares / K,
+//         x * (1 / sqrt(. + eps)) * weight with every product rounded to float32, then fp16 (the order of the
+//         additions of the sum of squares differs from the float32-butterfly kernel's, which can move 1 / sqrt by a
+//         float32 ulp); the weight row sits in LDS (ones when the norm has none);
+//   F6    the codes leave in the operand format of the 6-bit matrix instruction (gemm_f6.hip) -- q is then the encoded
+//         matrix of M rows, K-slab-major blocks of 96 bytes per 128 codes and row: a lane's 32 codes are one 24-byte piece.
+template <bool SPLIT, bool RMS = false, bool ADD = false, bool F6 = false>
 __global__ __launch_bounds__(256) void rotate_quant_mfma4096_kernel(const __half* __restrict__ x,
                                                                     uint8_t* __restrict__ q,
                                                                     __half* __restrict__ scales, uint32_t M,
-                                                                    float clip) {
+                                                                    float clip, const __half* __restrict__ add,
+                                                                    __half* __restrict__ sum_out,
+                                                                    const __half* __restrict__ weight, float eps) {
   const int lane = threadIdx.x & 63, col = lane & 31, h = lane >> 5;
   const uint32_t wave0 = blockIdx.x * 4u + (threadIdx.x >> 6), nwaves = gridDim.x * 4u;
+  __shared__ h8 wlds[RMS ? 512 : 1];                   // the norm weight, 16-byte chunk c = channels 8 c .. 8 c + 7
+  if constexpr (RMS) {
+    const h8 ones = {1, 1, 1, 1, 1, 1, 1, 1};
+    for (int i = threadIdx.x; i < 512; i += 256) wlds[i] = weight ? *(const h8*)(weight + 8 * i) : ones;
+    __syncthreads();
+  }
 
   // sign of H64[a][b] = parity(a & b).  Within a fragment only the low slot bits vary:
   // pattern over i times a per-fragment sign.
@@ -112,21 +129,55 @@ __global__ __launch_bounds__(256) void rotate_quant_mfma4096_kernel(const __half
 
   // The next row of this wave is requested before the current one is worked on: with two or three waves on a
   // SIMD nothing else would cover the two microseconds a row takes to arrive.
-  h8 xa[2][4], xn[2][4];
-  auto request = [&](uint32_t row, h8 (&dst)[2][4]) {
-    const __half* xr = x + (size_t)row * 4096;
+  h8 xa[2][4], xn[2][4], an[ADD ? 2 : 1][ADD ? 4 : 1];
+  auto request = [&](const __half* base, uint32_t row, auto& dst) {
+    const __half* xr = base + (size_t)row * 4096;
 #pragma unroll
     for (int jb = 0; jb < 2; ++jb)
 #pragma unroll
       for (int s = 0; s < 4; ++s) dst[jb][s] = *(const h8*)(xr + (32 * jb + col) * 64 + 16 * s + 8 * h);
   };
-  if (wave0 < M) request(wave0, xn);
+  if (wave0 < M) {
+    request(x, wave0, xn);
+    if constexpr (ADD) request(add, wave0, an);
+  }
   for (uint32_t row = wave0; row < M; row += nwaves) {
 #pragma unroll
     for (int jb = 0; jb < 2; ++jb)
 #pragma unroll
-      for (int s = 0; s < 4; ++s) xa[jb][s] = xn[jb][s];
-    if (row + nwaves < M) request(row + nwaves, xn);
+      for (int s = 0; s < 4; ++s) {
+        xa[jb][s] = xn[jb][s];
+        if constexpr (ADD) {
+          xa[jb][s] = __builtin_bit_cast(h8, add_h8(__builtin_bit_cast(v4i, xn[jb][s]), __builtin_bit_cast(v4i, an[jb][s])));
+          *(h8*)(sum_out + (size_t)row * 4096 + (32 * jb + col) * 64 + 16 * s + 8 * h) = xa[jb][s];
+        }
+      }
+    if (row + nwaves < M) {
+      request(x, row + nwaves, xn);
+      if constexpr (ADD) request(add, row + nwaves, an);
+    }
+    if constexpr (RMS) {
+      float ss = 0.f;
+#pragma unroll
+      for (int jb = 0; jb < 2; ++jb)
+#pragma unroll
+        for (int s = 0; s < 4; ++s)
+#pragma unroll
+          for (int i = 0; i < 8; ++i) ss = __builtin_fmaf((float)xa[jb][s][i], (float)xa[jb][s][i], ss);
+      ss = wave_sum(ss);
+      const float inv = 1.0f / __builtin_sqrtf(ss / 4096.0f + eps);
+#pragma unroll
+      for (int jb = 0; jb < 2; ++jb)
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+          const h8 g = wlds[(32 * jb + col) * 8 + 2 * s + h];
+          h8 y;
+#pragma unroll
+          for (int i = 0; i < 8; ++i)
+            y[i] = (_Float16)round_here(round_here((float)xa[jb][s][i] * inv) * (float)g[i]);
+          xa[jb][s] = y;
+        }
+    }
 
     v16f w[2][2];  // level-2 accumulators [t' tile][j' tile]
 #pragma unroll
@@ -196,7 +247,18 @@ __global__ __launch_bounds__(256) void rotate_quant_mfma4096_kernel(const __half
     for (int nt = 0; nt < 2; ++nt) {
       const v4i out = careful ? quantise_block<true>(y[0][nt], y[1][nt], rinv, hb)
                               : quantise_block<false>(y[0][nt], y[1][nt], rinv, hb);
-      *(v4i*)(qr + (32 * nt + col) * 32 + 16 * h) = out;
+      if constexpr (F6) {
+        // this lane: codes 32 h .. 32 h + 31 of block j' = 32 nt + col = the piece (h, j' % 2) of 128-code block j' / 2
+        const int jp = 32 * nt + col;
+        const unsigned long long c0 = bf6_of_nibbles((unsigned)out[0]), c1 = bf6_of_nibbles((unsigned)out[1]),
+                                 c2 = bf6_of_nibbles((unsigned)out[2]), c3 = bf6_of_nibbles((unsigned)out[3]);
+        v2i* dst = (v2i*)(q + ((size_t)(jp >> 1) * M + row) * kF6BlockBytes + 48 * h + 24 * (jp & 1));
+        dst[0] = v2i{(int)(unsigned)c0, (int)((unsigned)(c0 >> 32) | ((unsigned)c1 << 16))};
+        dst[1] = v2i{(int)(unsigned)(c1 >> 16), (int)(unsigned)c2};
+        dst[2] = v2i{(int)((unsigned)(c2 >> 32) | ((unsigned)c3 << 16)), (int)(unsigned)(c3 >> 16)};
+      } else {
+        *(v4i*)(qr + (32 * nt + col) * 32 + 16 * h) = out;
+      }
     }
     if (lane == 0) scales[row] = __builtin_bit_cast(__half, s16);
   }
@@ -624,6 +686,10 @@ int launch_rotate_quant_mfma_f6(const __half* x, uint8_t* encoded, __half* scale
   return fail(FLH_EINVAL, "rotate_quant_f6 (matrix-core mode): K = %u is not supported", K);
 }
 
+int launch_rotate_quant_mfma4096(const __half* x, const __half* add, __half* sum_out, bool rms, const __half* weight,
+                                 float eps, uint8_t* q, __half* scales, uint32_t M, float clip, bool f6,
+                                 hipStream_t stream);
+
 // launcher used by flh_rotate_quant_i4 (fwht_quant.hip)
 int launch_rotate_quant_mfma(const __half* x, uint8_t* q, __half* scales, uint32_t M, uint32_t K, float clip,
                              hipStream_t stream) {
@@ -631,9 +697,24 @@ int launch_rotate_quant_mfma(const __half* x, uint8_t* q, __half* scales, uint32
   if (K == 14336) return launch_dense<7>(x, q, scales, M, clip, stream);
   if (K != 4096) return fail(FLH_EINVAL, "rotate_quant (matrix-core mode): K = %u is not supported", K);
   // persistent waves (two workgroups of four per compute unit are resident): rows beyond the first are prefetched
+  return launch_rotate_quant_mfma4096(x, nullptr, nullptr, false, nullptr, 0.f, q, scales, M, clip, false, stream);
+}
+
+// K = 4096 on the matrix cores with the prologues / output format of the float32-butterfly kernels (used by the
+// entry points of fwht_quant.hip for FLH_HAD_MFMA): residual addition (add, sum_out: both or neither; with rms only),
+// RMSNorm (weight may be null), 6-bit operand output
+int launch_rotate_quant_mfma4096(const __half* x, const __half* add, __half* sum_out, bool rms, const __half* weight,
+                                 float eps, uint8_t* q, __half* scales, uint32_t M, float clip, bool f6,
+                                 hipStream_t stream) {
   const unsigned blocks = (M + 3) / 4 < 512u ? (M + 3) / 4 : 512u;
-  hipLaunchKernelGGL((rotate_quant_mfma4096_kernel<true>), dim3(blocks), dim3(256), 0, stream, x, q, scales, M, clip);
-  return check_launch("rotate_quant_mfma");
+  auto go = [&](auto kern) {
+    hipLaunchKernelGGL(kern, dim3(blocks), dim3(256), 0, stream, x, q, scales, M, clip, add, sum_out, weight, eps);
+    return check_launch("rotate_quant_mfma");
+  };
+  if (add && !rms) return fail(FLH_EINVAL, "rotate_quant (matrix-core mode): the residual addition comes with RMSNorm");
+  if (!rms) return f6 ? go(rotate_quant_mfma4096_kernel<true, false, false, true>) : go(rotate_quant_mfma4096_kernel<true>);
+  if (!add) return f6 ? go(rotate_quant_mfma4096_kernel<true, true, false, true>) : go(rotate_quant_mfma4096_kernel<true, true>);
+  return f6 ? go(rotate_quant_mfma4096_kernel<true, true, true, true>) : go(rotate_quant_mfma4096_kernel<true, true, true>);
 }
 
 }  // namespace flh

@@ -684,6 +684,9 @@ int launch_rotate_quant_mfma(const __half* x, uint8_t* q, __half* scales, uint32
 bool rotate_quant_mfma_supports(uint32_t K);
 int launch_silu_mul_rotate_quant_mfma(const __half* gate, const __half* up, uint8_t* q, __half* scales, uint32_t M,
                                       uint32_t K, hipStream_t stream);
+int launch_rotate_quant_mfma4096(const __half* x, const __half* add, __half* sum_out, bool rms, const __half* weight,
+                                 float eps, uint8_t* q, __half* scales, uint32_t M, float clip, bool f6,
+                                 hipStream_t stream);
 int launch_rotate_quant_mfma_f6(const __half* x, uint8_t* encoded, __half* scales, uint32_t M, uint32_t K, float clip,
                                 hipStream_t stream);
 
@@ -742,13 +745,19 @@ extern "C" int flh_rmsnorm_rotate_quant_i4(const flh_half* x, const flh_half* we
   if (misaligned16(x, q_packed)) return fail(FLH_EINVAL, "rmsnorm_rotate_quant: x and q_packed must be 16-byte aligned");
   if (!(clip_ratio > 0.f)) return fail(FLH_EINVAL, "rmsnorm_rotate_quant: clip_ratio must be positive");
   if (!(eps >= 0.f)) return fail(FLH_EINVAL, "rmsnorm_rotate_quant: eps must not be negative");
-  if (hadamard != FLH_HAD_NONE && hadamard != FLH_HAD_F32)
-    return fail(FLH_EINVAL, "rmsnorm_rotate_quant: hadamard mode must be FLH_HAD_NONE or FLH_HAD_F32");
+  if (hadamard != FLH_HAD_NONE && hadamard != FLH_HAD_F32 && hadamard != FLH_HAD_MFMA)
+    return fail(FLH_EINVAL, "rmsnorm_rotate_quant: unknown hadamard mode %d", hadamard);
   if (K % 512 || !is_pow2(K / 512) || K > 8192)
     return fail(FLH_EINVAL, "rmsnorm_rotate_quant: K (%u) must be 512, 1024, 2048, 4096 or 8192", K);
   if (M == 0) return FLH_OK;
   const __half *xh = (const __half*)x, *wh = (const __half*)weight;
   __half *sh = (__half*)scales, *yh = (__half*)y_out;
+  if (hadamard == FLH_HAD_MFMA) {                      // matrix cores: K = 4096 without y_out, else the float32 butterflies
+    if (K == 4096 && !yh && (!wh || !misaligned16(wh)))
+      return launch_rotate_quant_mfma4096(xh, nullptr, nullptr, true, wh, eps, q_packed, sh, M, clip_ratio, false,
+                                          (hipStream_t)stream);
+    hadamard = FLH_HAD_F32;
+  }
   const bool had = hadamard != FLH_HAD_NONE;
   hipStream_t st = (hipStream_t)stream;
   if (had && K == 4096 && !yh && clip_ratio >= 1.0f && M <= kRow8MaxRows && (!wh || !misaligned16(wh))) {
@@ -773,18 +782,22 @@ extern "C" int flh_add_rmsnorm_rotate_quant_i4(const flh_half* x, const flh_half
   if (weight && misaligned16(weight)) return fail(FLH_EINVAL, "add_rmsnorm_rotate_quant: weight must be 16-byte aligned");
   if (!(clip_ratio > 0.f)) return fail(FLH_EINVAL, "add_rmsnorm_rotate_quant: clip_ratio must be positive");
   if (!(eps >= 0.f)) return fail(FLH_EINVAL, "add_rmsnorm_rotate_quant: eps must not be negative");
-  if (hadamard != FLH_HAD_NONE && hadamard != FLH_HAD_F32)
-    return fail(FLH_EINVAL, "add_rmsnorm_rotate_quant: hadamard mode must be FLH_HAD_NONE or FLH_HAD_F32");
+  if (hadamard != FLH_HAD_NONE && hadamard != FLH_HAD_F32 && hadamard != FLH_HAD_MFMA)
+    return fail(FLH_EINVAL, "add_rmsnorm_rotate_quant: unknown hadamard mode %d", hadamard);
   if (K % 512 || !is_pow2(K / 512) || K > 8192)
     return fail(FLH_EINVAL, "add_rmsnorm_rotate_quant: K (%u) must be 512, 1024, 2048, 4096 or 8192", K);
   if (M == 0) return FLH_OK;
   const __half *xh = (const __half*)x, *ah = (const __half*)add, *wh = (const __half*)weight;
   __half *sh = (__half*)scales, *oh = (__half*)sum_out;
-  const bool had = hadamard != FLH_HAD_NONE;
   hipStream_t st = (hipStream_t)stream;
   // (the eight-waves-per-row kernel lets other waves read x and add after one has stored its part of the sum)
   if ((const void*)sum_out == (const void*)x || (const void*)sum_out == (const void*)add)
     return fail(FLH_EINVAL, "add_rmsnorm_rotate_quant: sum_out must not be x or add");
+  if (hadamard == FLH_HAD_MFMA) {                      // matrix cores: K = 4096, else the float32 butterflies
+    if (K == 4096) return launch_rotate_quant_mfma4096(xh, ah, oh, true, wh, eps, q_packed, sh, M, clip_ratio, false, st);
+    hadamard = FLH_HAD_F32;
+  }
+  const bool had = hadamard != FLH_HAD_NONE;
   if (had && K == 4096 && clip_ratio >= 1.0f && M <= kRow8MaxRows) {
     hipLaunchKernelGGL(add_rmsnorm_rotate_quant_row8_kernel, dim3(M), dim3(512), 0, st, xh, ah, oh, wh, eps, q_packed, sh,
                        1.0f / 64.0f);
@@ -818,8 +831,10 @@ extern "C" int flh_rotate_quant_f6(const flh_half* x, const flh_half* add, flh_h
   __half *sh = (__half*)scales, *oh = (__half*)sum_out;
   hipStream_t st = (hipStream_t)stream;
   if (hadamard == FLH_HAD_MFMA) {
-    if (rmsnorm) return fail(FLH_EINVAL, "%s: the matrix-core rotation has no RMSNorm prologue", who);
-    if (K != 11008 && K != 14336) return fail(FLH_EINVAL, "%s: matrix-core rotation with 6-bit output: K (%u) must be 11008 or 14336", who, K);
+    if (K == 4096) return launch_rotate_quant_mfma4096(xh, ah, oh, rmsnorm != 0, wh, eps, encoded, sh, M, clip_ratio, true, st);
+    if (rmsnorm) return fail(FLH_EINVAL, "%s: the matrix-core rotation has an RMSNorm prologue for K = 4096 only", who);
+    if (K != 11008 && K != 14336)
+      return fail(FLH_EINVAL, "%s: matrix-core rotation with 6-bit output: K (%u) must be 4096, 11008 or 14336", who, K);
     return launch_rotate_quant_mfma_f6(xh, encoded, sh, M, K, clip_ratio, st);
   }
   if (hadamard != FLH_HAD_NONE && hadamard != FLH_HAD_F32) return fail(FLH_EINVAL, "%s: unknown hadamard mode %d", who, hadamard);

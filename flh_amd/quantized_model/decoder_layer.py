@@ -126,6 +126,10 @@ class W4A4DecoderLayer(torch.nn.Module):
         self.act_group_size = act_group_size
         self.weight_group_size = weight_group_size
         self.record = None
+        # Token configuration, prefill-sized batches of the fused path: rotate rows of 4096 channels on the matrix cores
+        # instead of with float32 butterflies (codes one step apart from the exactly rounded transform in fewer than 1e-4 of
+        # the values -- closer to the float64 transform than the butterflies are -- for 5 us per launch at 4096 tokens).
+        self.fast_rotation = False
         kv = num_kv_heads * self.head_dim
         shapes = {"q_proj": (hidden_size, hidden_size), "k_proj": (hidden_size, kv), "v_proj": (hidden_size, kv),
                   "o_proj": (hidden_size, hidden_size), "gate_proj": (hidden_size, intermediate_size),
@@ -204,19 +208,26 @@ class W4A4DecoderLayer(torch.nn.Module):
         return (bool(consumers) and self.activation == "token" and self.fused and self.record is None
                 and width in self._F6_WIDTHS and all(l.wants_six_bit(n_rows) for l in consumers))
 
+    def _rotation_mode(self, rows, k):
+        """hadamard argument of the whole-row ops for `rows` rows of k channels."""
+        fast = self.fast_rotation and self.fused and self.record is None and k == 4096 and rows > 64
+        return "fast" if fast else True
+
     def _token_quant(self, stage, x, norm=None, norm_name=None, consumers=()):
         """Whole-row rotation + one scale per token (after RMSNorm when `norm` is given)."""
         rows = x.reshape(-1, x.size(-1)).contiguous()
+        mode = self._rotation_mode(rows.size(0), rows.size(1))
         if self._six_bit_for(consumers, rows.size(0), rows.size(1)):
             if norm is not None:
-                q, s = _ops().rotate_and_quantize_f6(rows, norm_weight=self._norm_weight16(norm_name, norm), eps=norm.eps)
+                q, s = _ops().rotate_and_quantize_f6(rows, hadamard=mode, norm_weight=self._norm_weight16(norm_name, norm),
+                                                     eps=norm.eps)
             else:
-                q, s = _ops().rotate_and_quantize_f6(rows)
+                q, s = _ops().rotate_and_quantize_f6(rows, hadamard=mode)
             return s.view(*x.shape[:-1], 1), None, q.view(*x.shape[:-1], -1)
         if norm is not None and self.fused:
-            q, s = _ops().rmsnorm_rotate_and_quantize_i4(rows, self._norm_weight16(norm_name, norm), norm.eps)
+            q, s = _ops().rmsnorm_rotate_and_quantize_i4(rows, self._norm_weight16(norm_name, norm), norm.eps, hadamard=mode)
         else:
-            q, s = _ops().rotate_and_quantize_i4(norm(rows) if norm is not None else rows, hadamard=True)
+            q, s = _ops().rotate_and_quantize_i4(norm(rows) if norm is not None else rows, hadamard=mode)
         self._tap(stage + ".input", rows)
         self._tap(stage + ".codes", q)
         self._tap(stage + ".scales", s)
@@ -245,13 +256,13 @@ class W4A4DecoderLayer(torch.nn.Module):
         k = x.size(-1)
         if k in (512, 1024, 2048, 4096, 8192) and self._six_bit_for(consumers, x.numel() // k, k):
             total, q, s = _ops().rotate_and_quantize_f6(
-                x.reshape(-1, k).contiguous(), norm_weight=self._norm_weight16(norm_name, norm), eps=norm.eps,
-                add=add.reshape(-1, k).contiguous())
+                x.reshape(-1, k).contiguous(), hadamard=self._rotation_mode(x.numel() // k, k),
+                norm_weight=self._norm_weight16(norm_name, norm), eps=norm.eps, add=add.reshape(-1, k).contiguous())
             return total.view(x.shape), s.view(*x.shape[:-1], 1), None, q.view(*x.shape[:-1], -1)
         if self.activation == "token" and self.fused and self.record is None and k in (512, 1024, 2048, 4096, 8192):
             total, q, s = _ops().add_rmsnorm_rotate_and_quantize_i4(
                 x.reshape(-1, k).contiguous(), add.reshape(-1, k).contiguous(), self._norm_weight16(norm_name, norm),
-                norm.eps)
+                norm.eps, hadamard=self._rotation_mode(x.numel() // k, k))
             return total.view(x.shape), s.view(*x.shape[:-1], 1), None, q.view(*x.shape[:-1], -1)
         x = x + add
         return (x,) + tuple(self._norm_quant(stage, norm, norm_name, quantizer, x, consumers))

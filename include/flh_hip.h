@@ -199,7 +199,7 @@ int flh_group_quant_f6(const flh_half* x, uint8_t* encoded, flh_half* scales, ui
  * encoded [M rows, K / 128 * 96 bytes] as flh_encode_f6 lays it out, scales [M].  hadamard FLH_HAD_NONE / FLH_HAD_F32 with
  * K = 512 .. 8192 a power of two, optionally with the prologues of flh_rmsnorm_rotate_quant_i4 (rmsnorm != 0; weight [K]
  * or null, eps) and flh_add_rmsnorm_rotate_quant_i4 (add / sum_out [M, K], both or neither, only with rmsnorm);
- * FLH_HAD_MFMA with K = 11008 / 14336 (no prologue).  The bytes equal flh_encode_f6 of the nibble output of the
+ * FLH_HAD_MFMA with K = 4096 (any prologue) or K = 11008 / 14336 (no prologue).  The bytes equal flh_encode_f6 of the nibble output of the
  * corresponding flh_*rotate_quant_i4 call, the scales are the same.  No counterpart in the reference. */
 int flh_rotate_quant_f6(const flh_half* x, const flh_half* add, flh_half* sum_out, int rmsnorm, const flh_half* weight,
                         float eps, uint8_t* encoded, flh_half* scales, uint32_t M, uint32_t K, int hadamard, float clip_ratio,
@@ -260,7 +260,9 @@ int flh_rmsnorm_group_quant_i4(const flh_half* x, const flh_half* weight, uint8_
  * RMSNorm.forward in torch, flh/nn/normalization.py:12-20, before its quantiser): x [M, K] fp16, weight [K] fp16 or
  * NULL, K in {512, 1024, 2048, 4096, 8192}; the fp16 row y = fp16(float(x) * rsqrt(sum x^2 / K + eps) [* weight]) is
  * then treated exactly as flh_rotate_quant_i4 treats its input (hadamard FLH_HAD_NONE or FLH_HAD_F32, one scale per
- * row, optional clip, optional y_out = the rotated row).  The float32 summation order is the device's. */
+ * row, optional clip, optional y_out = the rotated row).  The float32 summation order is the device's.
+ * hadamard FLH_HAD_MFMA: K = 4096 without y_out rotates on the matrix cores (not bit-exact, as for flh_rotate_quant_i4;
+ * other shapes take FLH_HAD_F32); the same holds for flh_add_rmsnorm_rotate_quant_i4 and flh_rotate_quant_f6. */
 int flh_rmsnorm_rotate_quant_i4(const flh_half* x, const flh_half* weight, float eps, uint8_t* q_packed,
                                 flh_half* scales, flh_half* y_out, uint32_t M, uint32_t K, int hadamard,
                                 float clip_ratio, void* stream);

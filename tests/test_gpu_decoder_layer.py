@@ -140,3 +140,33 @@ def test_token_layer_on_the_six_bit_path_gives_the_same_bits(six):
     short = x[:, :8].contiguous()                     # 16 rows: below the threshold, the int8 / decode kernels
     cs, ss = rotary_tables(torch.arange(8, device="cuda"), 128)
     assert torch.equal(plain(short, cs, ss)[0], fast(short, cs, ss)[0])
+
+
+def test_fast_rotation_option_changes_almost_nothing():
+    """fast_rotation=True: rows of 4096 channels rotate on the matrix cores in the fused prefill path.  Codes differ from the
+    float32-butterfly launches in fewer than 1e-4 of the values (tests/test_gpu_rotate_f6.py), so the layer's update moves
+    by far less than its int4 noise; the decode path (a single token) stays on the bit-exact kernels."""
+    import math
+    from flh_amd.quantized_model import W4A4DecoderLayer, rotary_tables
+    torch.manual_seed(3)
+    hidden, inter, heads = 4096, 1024, 32
+    dims = {"q_proj": (hidden, hidden), "k_proj": (hidden, hidden), "v_proj": (hidden, hidden), "o_proj": (hidden, hidden),
+            "gate_proj": (inter, hidden), "up_proj": (inter, hidden), "down_proj": (hidden, inter)}
+    w = {n: (torch.randn(s, device="cuda") / math.sqrt(s[1])).half() for n, s in dims.items()}
+    for six in (False, None):
+        layer = W4A4DecoderLayer.from_float(w, heads, heads, fused=True, activation="token", weight_group_size=128, six_bit=six)
+        x = torch.randn(2, 160, hidden, device="cuda").half()
+        cos, sin = rotary_tables(torch.arange(160, device="cuda"), 128)
+        print(f"case layer fast rotation six_bit={six}", flush=True)
+        with torch.no_grad():
+            y0, (k0, v0) = layer(x, cos, sin)
+            layer.fast_rotation = True
+            y1, (k1, v1) = layer(x, cos, sin)
+            rel = ((y1.float() - y0.float()).norm() / (y0.float() - x.float()).norm()).item()
+            print(f"  relative difference of the layer's update {rel:.2e}", flush=True)
+            assert 0 < rel < 2e-2
+            # one token: the same launches with or without the option
+            d1, _ = layer(x[:, :1].contiguous(), cos[:1], sin[:1])
+            layer.fast_rotation = False
+            d0, _ = layer(x[:, :1].contiguous(), cos[:1], sin[:1])
+            assert torch.equal(d0, d1)

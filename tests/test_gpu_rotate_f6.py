@@ -90,3 +90,48 @@ def test_argument_errors(ops):
         ops.rotate_and_quantize_f6(torch.zeros(4, 11008, dtype=torch.float16, device="cuda"), eps=1e-5)
     with pytest.raises(RuntimeError):
         ops.rotate_and_quantize_f6(x.float())
+
+
+def _unpack(q):
+    """[M, K/2] u8 -> signed codes [M, K] int32 (low nibble first)"""
+    b = q.to(torch.int32)
+    lo, hi = b & 15, b >> 4
+    c = torch.stack((lo, hi), dim=-1).reshape(q.size(0), -1)
+    return torch.where(c > 7, c - 16, c)
+
+
+@pytest.mark.parametrize("m", [3, 300, 2048])
+@pytest.mark.parametrize("prologue", ["none", "rms", "rms_weight", "add_rms_weight"])
+def test_matrix_core_rotation_of_4096_with_prologues(ops, m, prologue):
+    """hadamard="fast" at K = 4096 behind RMSNorm / the residual addition, nibble and 6-bit output: not bit-exact by
+    design (the matrix cores sum in their own order; the sum of squares of the norm too), so measured against the
+    float32-butterfly launches -- codes one step apart at a rate below 1e-4, scales at most one fp16 step apart in a
+    few rows per thousand; the residual sum is the same bits; the 6-bit output is the encoding of the same mode's
+    nibble output, byte for byte."""
+    k = 4096
+    print(f"case fast 4096 m={m} {prologue}", flush=True)
+    x = dev(syn.activations(m, k, seed=5 * m + 1))
+    add = dev((np.random.default_rng(m).standard_normal((m, k)) * 0.4).astype(np.float16)) if prologue.startswith("add") else None
+    w = dev(np.random.default_rng(2).uniform(0.5, 1.5, k).astype(np.float16)) if "weight" in prologue else None
+    if prologue == "none":
+        q, s = ops.rotate_and_quantize_i4(x, hadamard="fast")
+        qe, se = ops.rotate_and_quantize_i4(x, hadamard="exact")
+        enc, s6 = ops.rotate_and_quantize_f6(x, hadamard="fast")
+    elif add is None:
+        q, s = ops.rmsnorm_rotate_and_quantize_i4(x, w, 1e-5, hadamard="fast")
+        qe, se = ops.rmsnorm_rotate_and_quantize_i4(x, w, 1e-5, hadamard="exact")
+        enc, s6 = ops.rotate_and_quantize_f6(x, hadamard="fast", norm_weight=w, eps=1e-5)
+    else:
+        total, q, s = ops.add_rmsnorm_rotate_and_quantize_i4(x, add, w, 1e-5, hadamard="fast")
+        total_e, qe, se = ops.add_rmsnorm_rotate_and_quantize_i4(x, add, w, 1e-5, hadamard="exact")
+        total6, enc, s6 = ops.rotate_and_quantize_f6(x, hadamard="fast", norm_weight=w, eps=1e-5, add=add)
+        assert torch.equal(total, total_e) and torch.equal(total6, total_e)       # the residual stream: the same bits
+    diff = (_unpack(q) - _unpack(qe)).abs()
+    s_step = (s.view(torch.int16).int() - se.view(torch.int16).int()).abs()
+    print(f"  code mismatch rate {(diff != 0).float().mean().item():.2e}, scale mismatch rate "
+          f"{(s_step != 0).float().mean().item():.2e}", flush=True)
+    assert int(diff.max()) <= 1 and (diff != 0).float().mean().item() < 1e-4
+    assert int(s_step.max()) <= 1 and (s_step != 0).float().mean().item() <= max(5e-3, 1.0 / m if m < 10 else 0)
+    # the 6-bit output of the same mode: byte for byte the encoding of its nibble output
+    assert torch.equal(s6.view(torch.int16), s.view(torch.int16))
+    assert torch.equal(enc, ops.encode_f6(q))
