@@ -38,6 +38,10 @@ typedef __attribute__((address_space(3))) s4 lds_s4;
 
 // byte offset inside a tile of the 16-byte chunk `c` (8 channels) of key row `r`
 __device__ __forceinline__ int chunk_at(int r, int c) { return r * (kHeadDim * 2) + ((c ^ (r & 15)) << 4); }
+// the same for a V tile, whose swizzle serves the transpose loads: one of them reads 64 bytes (four chunks) of each of
+// four consecutive rows, which must fall into four different quarters of the 256-byte bank line
+__device__ __forceinline__ int v_swizzle(int r) { return (r & 3) << 2; }
+__device__ __forceinline__ int v_chunk_at(int r, int c) { return r * (kHeadDim * 2) + ((c ^ v_swizzle(r)) << 4); }
 
 __global__ __launch_bounds__(256, 2) void prefill_attention_kernel(const __half* __restrict__ q,
                                                                    const __half* __restrict__ k_cache,
@@ -82,11 +86,11 @@ __global__ __launch_bounds__(256, 2) void prefill_attention_kernel(const __half*
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int inst = wave * 4 + i;                   // 0 .. 15
-      const int r = inst * 4 + (lane >> 4), c = (lane & 15) ^ (r & 15);
+      const int r = inst * 4 + (lane >> 4);
       const int key = min(step * kKeysPerStep + r, total_keys - 1);
-      const size_t off = (size_t)key * kHeadDim + c * 8;
-      load_to_lds16(kbase + off, lds0 + buf * kTileBytes + inst * 1024);
-      load_to_lds16(vbase + off, lds0 + (2 + buf) * kTileBytes + inst * 1024);
+      const size_t row = (size_t)key * kHeadDim;
+      load_to_lds16(kbase + row + ((lane & 15) ^ (r & 15)) * 8, lds0 + buf * kTileBytes + inst * 1024);
+      load_to_lds16(vbase + row + ((lane & 15) ^ v_swizzle(r)) * 8, lds0 + (2 + buf) * kTileBytes + inst * 1024);
     }
   };
 
@@ -186,8 +190,8 @@ __global__ __launch_bounds__(256, 2) void prefill_attention_kernel(const __half*
 #pragma unroll
         for (int dt = 0; dt < 4; ++dt) {
           const int c = 4 * dt + tr_chunk0;
-          const s4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4*)(vt_lds + chunk_at(row0, c) + tr_half));
-          const s4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4*)(vt_lds + chunk_at(row0 + 8, c) + tr_half));
+          const s4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4*)(vt_lds + v_chunk_at(row0, c) + tr_half));
+          const s4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4*)(vt_lds + v_chunk_at(row0 + 8, c) + tr_half));
           const h8 a = __builtin_bit_cast(h8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
           o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, pb[kt][ks], o[dt], 0, 0, 0);
         }
