@@ -6,7 +6,8 @@
 // layout the quantiser of o_proj reads.
 //
 // One workgroup = 4 waves = 128 consecutive queries of one head, 32 per wave; keys in blocks of 64, K and V tiles
-// double-buffered in LDS by direct-to-LDS loads (row-major, 16-byte chunks XOR-swizzled by the row).  Both products run
+// double-buffered in LDS by direct-to-LDS loads (row-major, 16-byte chunks XOR-swizzled by the row; the V tile has a
+// swizzle of its own for the transpose loads).  Both products run
 // on v_mfma_f32_32x32x16_f16 in transposed form, so that a lane owns one query throughout:
 //
 //   S^T[key, query] = sum_d K[key, d] Q[query, d]         A = K tile rows from LDS, B = the wave's queries (registers)
