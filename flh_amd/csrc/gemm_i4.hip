@@ -690,6 +690,10 @@ int launch(GemmArgs a, hipStream_t stream) {
   return check_launch("gemm_i4");
 }
 
+// More 256 x 128 tiles than compute units: do 128 x 128 tiles spread evenly what the large ones spread unevenly?  The
+// busiest of 256 compute units decides; it finishes a small tile in 0.575 of the time of a large one (measured).
+bool prefers_small_tiles(long t256, long t128) { return 0.575 * (double)((t128 + 255) / 256) < (double)((t256 + 255) / 256); }
+
 #ifndef FLH_GEMM_STAGES
 #define FLH_GEMM_STAGES 3
 #endif
@@ -705,13 +709,21 @@ int launch_by_shape(const GemmArgs& a, hipStream_t stream) {
   const int n_all = total_n(a);
   auto tiles = [&](int bm, int bn) { return (long)((a.M + bm - 1) / bm) * ((n_all + bn - 1) / bn); };
   const int kt = a.K >> 7;
-  // measured on the Llama shapes at M = 2048: with more large tiles than compute units the 256 x 128 tile wins
-  // (two workgroups share a compute unit); with at most one per compute unit a long K prefers the large tile
-  // split over two quads, a short K the 128 x 128 tile without any split
-  int tile = tiles(256, 128) > 256 ? 256 : tiles(128, 128) >= 256 ? (kt >= 64 ? 256 : 128) : 64;
+  // measured on the Llama shapes at M = 128 ... 4096 (256 compute units): with more large tiles than compute units the
+  // 256 x 128 tile wins (two workgroups share a compute unit) unless 128 x 128 tiles spread evenly what it spreads
+  // unevenly (a compute unit finishes a small tile in 0.575 of the time of a large one); with at most one large tile per
+  // compute unit a long K prefers the large tile split over two quads as soon as the 128 x 128 tiles would come two to a
+  // compute unit, else the 128 x 128 tile (split over two quads when there is at most one per compute unit and K is
+  // long); below 160 such tiles the 64 x 64 tile with its K splits
+  const long t256 = tiles(256, 128), t128 = tiles(128, 128);
+  int tile;
+  if (t256 > 256) tile = prefers_small_tiles(t256, t128) ? 128 : 256;
+  else if (t128 >= 256) tile = kt >= 64 && t128 > 256 ? 256 : 128;
+  else tile = t128 >= 160 ? 128 : 64;
   if (env_tile == 256 || env_tile == 128 || env_tile == 64) tile = env_tile;
-  const long n_tiles = tile == 256 ? tiles(256, 128) : tile == 128 ? tiles(128, 128) : tiles(64, 64);
-  int ks = tile == 256 ? (n_tiles <= 256 ? 2 : 1) : tile == 128 ? 1 : n_tiles <= 256 ? 4 : n_tiles <= 512 ? 2 : 1;
+  const long n_tiles = tile == 256 ? t256 : tile == 128 ? t128 : tiles(64, 64);
+  int ks = tile == 256 ? (n_tiles <= 256 ? 2 : 1)
+                       : tile == 128 ? (n_tiles <= 256 && kt >= 64 ? 2 : 1) : n_tiles <= 256 ? 4 : n_tiles <= 512 ? 2 : 1;
   if (env_ks == 1 || env_ks == 2 || env_ks == 4) ks = env_ks;
   if (ks == 4 && tile != 64) ks = 2;
   while (ks > 1 && kt / ks < 2) ks >>= 1;
@@ -764,7 +776,7 @@ int gemm_dispatch(GemmArgs a, int epi, int group, hipStream_t stream) {
 template <int EPI>
 int launch_swiglu(const GemmArgs& a, int group, hipStream_t stream) {
   auto tiles = [&](int bm) { return (long)((a.M + bm - 1) / bm) * ((a.N + 63) / 64); };
-  int tile = tiles(256) > 256 ? 256 : tiles(128) >= 256 ? 128 : 64;
+  int tile = tiles(256) > 256 ? (prefers_small_tiles(tiles(256), tiles(128)) ? 128 : 256) : tiles(128) >= 160 ? 128 : 64;
   const int forced = g_tune_tile.load(std::memory_order_relaxed);
   if (forced == 256 || forced == 128 || forced == 64) tile = forced;
   if constexpr (EPI == kRowScale) {
@@ -781,8 +793,8 @@ int launch_swiglu(const GemmArgs& a, int group, hipStream_t stream) {
 // q / k / v launches with the rotary embedding and the cache write in the epilogue: 128-column tiles only
 template <int EPI>
 int launch_qkv_rope(const GemmArgs& a, hipStream_t stream) {
-  const long tiles256 = (long)((a.M + 255) / 256) * (total_n(a) / 128);
-  int tile = tiles256 > 256 ? 256 : 128;
+  const long tiles256 = (long)((a.M + 255) / 256) * (total_n(a) / 128), tiles128 = (long)((a.M + 127) / 128) * (total_n(a) / 128);
+  int tile = tiles256 > 256 && !prefers_small_tiles(tiles256, tiles128) ? 256 : 128;
   const int forced = g_tune_tile.load(std::memory_order_relaxed);
   if (forced == 256 || forced == 128) tile = forced;
   if constexpr (EPI == kRowScale) {                    // (the group epilogues have one thread per scale row: 128 x 128 only)
