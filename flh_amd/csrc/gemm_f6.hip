@@ -535,7 +535,10 @@ template <int EPI>
 int launch_f6_grouped(const GemmArgs& a, hipStream_t stream) {
   const int n_all = total_n_f6(a);
   auto tiles = [&](int bm, int bn) { return (long)((a.M + bm - 1) / bm) * ((n_all + bn - 1) / bn); };
-  if (tiles(128, 128) >= 200) return launch_f6<128, 128, 64, 64, 3, EPI>(a, stream);
+  int tile = tiles(128, 128) >= 200 ? 128 : 64;
+  const int forced = g_tune_tile.load(std::memory_order_relaxed);
+  if (forced == 128 || forced == 64) tile = forced;
+  if (tile == 128) return launch_f6<128, 128, 64, 64, 3, EPI>(a, stream);
   return launch_f6<64, 64, 32, 32, 3, EPI>(a, stream);
 }
 
