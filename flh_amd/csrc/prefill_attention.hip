@@ -109,6 +109,10 @@ __global__ __launch_bounds__(256, 2) void prefill_attention_kernel(const __half*
   const int tr_key = gi >> 2;                          // + key0 of the load
   const int tr_half = (gi & 1) << 3;                   // byte inside the 16-byte chunk
   const int tr_chunk0 = ((grp & 1) << 1) + ((gi & 3) >> 1);   // + 4 dt: chunk of 8 channels inside the row
+  // the lane's part of a transpose-load address for channel tile dt (the key rows of a load add a constant to it)
+  int tr_off[4];
+#pragma unroll
+  for (int dt = 0; dt < 4; ++dt) tr_off[dt] = v_chunk_at(4 * (grp >> 1) + tr_key, 4 * dt + tr_chunk0) + tr_half;
 
   issue(0, 0);
   for (int step = 0; step < n_steps; ++step) {
@@ -148,13 +152,19 @@ __global__ __launch_bounds__(256, 2) void prefill_attention_kernel(const __half*
     const int key0 = step * kKeysPerStep + 4 * h;
     const bool diagonal = __builtin_amdgcn_readfirstlane(step * kKeysPerStep + kKeysPerStep - 1 > past + q_first);
     float mx = -INFINITY;
+    if (diagonal) {                                    // (a branch of its own: most steps carry no mask arithmetic at all;
+      asm volatile("" ::: "memory");                   //  the empty statement keeps the compiler from predicating it)
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+          if (key0 + 32 * kt + 8 * (r >> 2) + (r & 3) > q_limit) st[kt][r] = -INFINITY;
+    }
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        if (diagonal && key0 + 32 * kt + 8 * (r >> 2) + (r & 3) > q_limit) st[kt][r] = -INFINITY;
-        mx = fmaxf(mx, st[kt][r]);
-      }
+      for (int r = 0; r < 16; ++r) mx = fmaxf(mx, st[kt][r]);
     mx = fmaxf(mx, lane_xor_f<32>(mx)) * scale_log2;   // (the scale is positive: the maximum commutes with it)
     const float m_new = fmaxf(m_run, mx);              // finite from the first step on: slot 0 is visible to every query
     float sum = 0.f;
@@ -187,12 +197,12 @@ __global__ __launch_bounds__(256, 2) void prefill_attention_kernel(const __half*
 #pragma unroll
       for (int ks = 0; ks < 2; ++ks) {
         // this half-wave's slots 8 h .. 8 h + 7 are keys 32 kt + 16 ks + 4 h + {0..3} and + 8 + {0..3}
-        const int row0 = 32 * kt + 16 * ks + 4 * (grp >> 1) + tr_key;
+        // (rows 32 kt + 16 ks and + 8 on: multiples of four, which the V swizzle does not see)
 #pragma unroll
         for (int dt = 0; dt < 4; ++dt) {
-          const int c = 4 * dt + tr_chunk0;
-          const s4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4*)(vt_lds + v_chunk_at(row0, c) + tr_half));
-          const s4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4*)(vt_lds + v_chunk_at(row0 + 8, c) + tr_half));
+          const uint8_t* at = vt_lds + tr_off[dt] + (32 * kt + 16 * ks) * (kHeadDim * 2);
+          const s4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4*)at);
+          const s4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4*)(at + 8 * (kHeadDim * 2)));
           const h8 a = __builtin_bit_cast(h8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
           o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, pb[kt][ks], o[dt], 0, 0, 0);
         }
