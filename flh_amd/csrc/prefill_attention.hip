@@ -82,16 +82,35 @@ __global__ __launch_bounds__(256, 2) void prefill_attention_kernel(const __half*
   const __half* vbase = v_cache + ((size_t)b * Hkv + hkv) * (size_t)max_len * kHeadDim;
   const unsigned lds0 = (unsigned)(size_t)lds;
 
-  // one load instruction moves four key rows (1 KiB); a wave issues four for K and four for V per step
-  auto issue = [&](int step, int buf) {
+  // one load instruction moves four key rows (1 KiB); a wave issues four for K and four for V per step.  A full step
+  // takes its rows from a wave-uniform base (the step's first key) plus per-lane byte offsets that never change; the
+  // last step of a sequence may run past the end and clamps its rows.
+  unsigned k_off[4], v_off[4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int inst = wave * 4 + i;                   // 0 .. 15
-      const int r = inst * 4 + (lane >> 4);
-      const int key = min(step * kKeysPerStep + r, total_keys - 1);
-      const size_t row = (size_t)key * kHeadDim;
-      load_to_lds16(kbase + row + ((lane & 15) ^ (r & 15)) * 8, lds0 + buf * kTileBytes + inst * 1024);
-      load_to_lds16(vbase + row + ((lane & 15) ^ v_swizzle(r)) * 8, lds0 + (2 + buf) * kTileBytes + inst * 1024);
+  for (int i = 0; i < 4; ++i) {
+    const int r = (wave * 4 + i) * 4 + (lane >> 4);
+    k_off[i] = (unsigned)(r * kHeadDim + ((lane & 15) ^ (r & 15)) * 8) * 2;
+    v_off[i] = (unsigned)(r * kHeadDim + ((lane & 15) ^ v_swizzle(r)) * 8) * 2;
+  }
+  auto issue = [&](int step, int buf) {
+    const int first = step * kKeysPerStep;
+    if (first + kKeysPerStep <= total_keys) {
+      const __half* kb = kbase + (size_t)first * kHeadDim;
+      const __half* vb = vbase + (size_t)first * kHeadDim;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        load_to_lds16(kb, k_off[i], lds0 + buf * kTileBytes + (wave * 4 + i) * 1024);
+        load_to_lds16(vb, v_off[i], lds0 + (2 + buf) * kTileBytes + (wave * 4 + i) * 1024);
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int inst = wave * 4 + i;                 // 0 .. 15
+        const int r = inst * 4 + (lane >> 4);
+        const size_t row = (size_t)min(first + r, total_keys - 1) * kHeadDim;
+        load_to_lds16(kbase + row + ((lane & 15) ^ (r & 15)) * 8, lds0 + buf * kTileBytes + inst * 1024);
+        load_to_lds16(vbase + row + ((lane & 15) ^ v_swizzle(r)) * 8, lds0 + (2 + buf) * kTileBytes + inst * 1024);
+      }
     }
   };
 
