@@ -194,6 +194,33 @@ def main():
                 break
             prev = ms
 
+    def engine_clock_under_load(seconds=1.5):
+        """The engine clock (MHz) the part sustains while the step's largest GEMM runs back to back, as rocm-smi reports
+        it from a second thread (None where the tool or the reading is not available): under dense matrix work these
+        parts settle well below the 2400 MHz the published peak is quoted at, and the fraction of that peak inherits it."""
+        import re
+        import subprocess
+        import threading
+        reading = [None]
+
+        def sample():
+            time.sleep(seconds * 0.5)
+            try:
+                out = subprocess.run(["rocm-smi", "--showclocks"], capture_output=True, text=True, timeout=30).stdout
+                m = re.search(r"sclk clock level: \d+: \((\d+)Mhz\)", out)
+                reading[0] = int(m.group(1)) if m else None
+            except Exception:
+                reading[0] = None
+        th = threading.Thread(target=sample)
+        th.start()
+        t0 = time.perf_counter()
+        while time.perf_counter() - t0 < seconds:
+            for _ in range(100):
+                ops.gemm_i4_dequant_o16(warm_q, weights["gate"][0], warm_s, weights["gate"][1])
+            torch.cuda.synchronize()
+        th.join()
+        return reading[0]
+
     def run_form(form):
         """(ms per step over exactly --steps steps after --warmup, median us per launch from a second pass with HIP
         events on the launch stream around every launch)"""
@@ -221,6 +248,7 @@ def main():
     # settle for longer than a handful of warm-up steps), which would otherwise be charged to whichever form is timed first
     ms_other, med_other = run_form(other_form)
     ms_per_step, med = run_form(args.launches)      # the headline: --warmup untimed steps, then exactly --steps timed ones
+    sclk = engine_clock_under_load()
     step = make_step("seven")
 
     # The same step with the weights of projections that share an input stored concatenated ([q; k; v] and
@@ -876,6 +904,9 @@ def main():
                      "traffic": GEMM_TRAFFIC_BYTES[args.launches] if M == 2048 else None,
                      "avg_launch_us": round(gemm_us / len(launches), 2),
                      "per_launch": launch_table(args.launches, med),
+                     # what the part clocks at under this load, and the fraction of the peak at that clock
+                     "engine_MHz_under_gemm_load": sclk,
+                     "frac_of_peak_at_that_clock": (round(gemm_tops / (PEAK_INT8_TOPS * sclk / 2400.0), 4) if sclk else None),
                      },
         f"launches={other_form}": {"us_per_layer": round(ms_other * 1e3, 1),
                                    "TOPS": round(total_ops / (ms_other * 1e-3) / 1e12, 2),
