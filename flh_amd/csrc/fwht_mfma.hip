@@ -91,7 +91,7 @@ __device__ __forceinline__ v4i quantise_block(const unsigned (&y0)[8], const uns
 //   F6    the codes leave in the operand format of the 6-bit matrix instruction (gemm_f6.hip) -- q is then the encoded
 //         matrix of M rows, K-slab-major blocks of 96 bytes per 128 codes and row: a lane's 32 codes are one 24-byte piece.
 template <bool SPLIT, bool RMS = false, bool ADD = false, bool F6 = false>
-__global__ __launch_bounds__(256) void rotate_quant_mfma4096_kernel(const __half* __restrict__ x,
+__global__ __launch_bounds__(256, 2) void rotate_quant_mfma4096_kernel(const __half* __restrict__ x,
                                                                     uint8_t* __restrict__ q,
                                                                     __half* __restrict__ scales, uint32_t M,
                                                                     float clip, const __half* __restrict__ add,
