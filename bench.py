@@ -194,8 +194,8 @@ def main():
                 break
             prev = ms
 
-    def engine_clock_under_load(seconds=1.5):
-        """The engine clock (MHz) the part sustains while the step's largest GEMM runs back to back, as rocm-smi reports
+    def engine_clock_under_load(lead=0.5, limit=20.0):
+        """The engine clock (MHz) the part sustains while one of the step's GEMMs runs back to back, as rocm-smi reports
         it from a second thread (None where the tool or the reading is not available): under dense matrix work these
         parts settle well below the 2400 MHz the published peak is quoted at, and the fraction of that peak inherits it."""
         import re
@@ -204,7 +204,7 @@ def main():
         reading = [None]
 
         def sample():
-            time.sleep(seconds * 0.5)
+            time.sleep(lead)
             try:
                 out = subprocess.run(["rocm-smi", "--showclocks"], capture_output=True, text=True, timeout=30).stdout
                 m = re.search(r"sclk clock level: \d+: \((\d+)Mhz\)", out)
@@ -214,7 +214,7 @@ def main():
         th = threading.Thread(target=sample)
         th.start()
         t0 = time.perf_counter()
-        while time.perf_counter() - t0 < seconds:
+        while th.is_alive() and time.perf_counter() - t0 < limit:    # the load lasts as long as the reading takes
             for _ in range(100):
                 ops.gemm_i4_dequant_o16(warm_q, weights["gate"][0], warm_s, weights["gate"][1])
             torch.cuda.synchronize()
