@@ -19,6 +19,8 @@ gemm_i4_dequant_o16 = _ext.gemm_i4_dequant_o16
 gemm_i4_dequant_o16_gs = _ext.gemm_i4_dequant_o16_gs
 gemm_i4_dequant_multi = _ext.gemm_i4_dequant_multi
 gemm_i4_swiglu = _ext.gemm_i4_swiglu
+gemm_i4_dequant_add = _ext.gemm_i4_dequant_add
+prefill_attention = _ext.prefill_attention
 rope_kv_cache_ = _ext.rope_kv_cache_
 rotate_quantize_gemm_i4 = _ext.rotate_quantize_gemm_i4
 rotate_quantize_gemm_i4_multi = _ext.rotate_quantize_gemm_i4_multi

@@ -14,6 +14,7 @@
 #include <ATen/hip/impl/HIPGuardImplMasqueradingAsCUDA.h>
 #include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
 
+#include <cmath>
 #include <mutex>
 #include <vector>
 
@@ -108,6 +109,48 @@ Tensor gemm_i4_dequant_o16_gs(const Tensor& A, const Tensor& B, const Tensor& A_
   TORCH_CHECK(A_scale.size(1) == K / group_size, "A_scale.shape[1] must equal K/group_size");
   TORCH_CHECK(B_scale.size(1) == K / group_size, "B_scale.shape[1] must equal K/group_size");
   return gemm_checked(A, B, A_scale, B_scale, group_size);
+}
+
+// fp16(residual + gemm): a decoder layer's residual addition in the GEMM's epilogue; `out` may be the residual itself
+Tensor gemm_i4_dequant_add(const Tensor& A, const Tensor& B, const Tensor& A_scale, const Tensor& B_scale,
+                           const Tensor& residual, int64_t group_size, const c10::optional<Tensor>& out) {
+  check_gemm_inputs(A, B, A_scale, B_scale);
+  const int64_t M = A.size(0), N = B.size(0), K = A.size(1) * 2;
+  auto shaped = [&](const Tensor& t, const char* what) {
+    TORCH_CHECK(t.is_cuda() && t.scalar_type() == torch::kFloat16 && t.is_contiguous() && t.device() == A.device(), what,
+                " must be a contiguous float16 CUDA tensor on the operands' device");
+    TORCH_CHECK(t.numel() == M * N && t.dim() >= 1 && t.size(-1) == N, what, " must have the shape of the output");
+  };
+  shaped(residual, "the residual");
+  if (out.has_value()) shaped(*out, "out");
+  Tensor D = out.has_value() ? *out : torch::empty({M, N}, A_scale.options());
+  if (M == 0 || N == 0) return D;
+  Launch l(A);
+  ok(flh_gemm_i4_add_o16(u8(A), u8(B), h(A_scale), h(B_scale), h(residual), hm(D), M, N, K, (int)A_scale.size(1),
+                         (int)B_scale.size(1), (int)group_size, stream_of(A)));
+  return D;
+}
+
+// causal attention of a block of new tokens over a cache (heads of 128 channels, grouped queries)
+Tensor prefill_attention(const Tensor& q, const Tensor& k_cache, const Tensor& v_cache, int64_t past,
+                         const c10::optional<double>& scale) {
+  for (const Tensor* t : {&q, &k_cache, &v_cache})
+    TORCH_CHECK(t->is_cuda() && t->scalar_type() == torch::kFloat16 && t->is_contiguous() && t->device() == q.device(),
+                "tensors must be contiguous float16 CUDA tensors on one device");
+  TORCH_CHECK(q.dim() == 4 && k_cache.dim() == 4 && k_cache.sizes() == v_cache.sizes() && k_cache.size(0) == q.size(0) &&
+                  k_cache.size(3) == q.size(3),
+              "q [B, T, Hq, d] and caches [B, Hkv, max_len, d] expected");
+  const int64_t B = q.size(0), T = q.size(1), Hq = q.size(2), d = q.size(3), Hkv = k_cache.size(1), max_len = k_cache.size(2);
+  TORCH_CHECK(d == 128, "head_dim must be 128");
+  TORCH_CHECK(Hkv > 0 && Hq % Hkv == 0, "Hq must be a multiple of Hkv");
+  TORCH_CHECK(past >= 0 && past + T <= max_len, "past + T must fit the cache");
+  Tensor out = torch::empty({B, T, Hq * d}, q.options());
+  if (B == 0 || T == 0) return out;
+  Launch l(q);
+  ok(flh_prefill_attention_f16(h(q), h(k_cache), h(v_cache), hm(out), (uint32_t)B, (uint32_t)T, (uint32_t)Hq, (uint32_t)Hkv,
+                               (uint32_t)d, (uint32_t)past, (uint32_t)max_len,
+                               (float)(scale.has_value() ? *scale : 1.0 / std::sqrt((double)d)), stream_of(q)));
+  return out;
 }
 
 // gate and up projection of a SwiGLU MLP in one launch: fp16(fp16(silu(gate)) * up)
@@ -418,6 +461,10 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         py::arg("B_scales"), py::arg("group_size") = 128);
   m.def("gemm_i4_swiglu", &gemm_i4_swiglu, py::arg("A"), py::arg("B_gate"), py::arg("B_up"), py::arg("A_scale"),
         py::arg("gate_scale"), py::arg("up_scale"), py::arg("group_size") = 128);
+  m.def("gemm_i4_dequant_add", &gemm_i4_dequant_add, py::arg("A"), py::arg("B"), py::arg("A_scale"), py::arg("B_scale"),
+        py::arg("residual"), py::arg("group_size") = 128, py::arg("out") = py::none());
+  m.def("prefill_attention", &prefill_attention, py::arg("q"), py::arg("k_cache"), py::arg("v_cache"), py::arg("past"),
+        py::arg("scale") = py::none());
   m.def("rotate_quantize_gemm_i4", &rotate_quantize_gemm_i4, py::arg("x"), py::arg("B"), py::arg("B_scale"));
   m.def("rotate_quantize_gemm_i4_multi", &rotate_quantize_gemm_i4_multi, py::arg("x"), py::arg("Bs"), py::arg("B_scales"));
   m.def("rope_kv_cache_", &rope_kv_cache_, py::arg("q"), py::arg("k"), py::arg("v"), py::arg("cos"), py::arg("sin"),

@@ -88,6 +88,37 @@ def test_decode_gemm_with_quantiser_inside_equal_ctypes(ext):
     assert same(ext.rotate_quantize_gemm_i4_multi(x, bs, ss), _ops.rotate_quantize_gemm_i4_multi(x, bs, ss))
 
 
+def test_residual_gemm_and_prefill_attention_equal_ctypes(ext):
+    rng = np.random.default_rng(11)
+    m, n, k = 300, 264, 512
+    print("case ext residual gemm / prefill attention", flush=True)
+    a = dev(syn.pack_codes(rng.integers(-8, 8, size=(m, k), dtype=np.int8)))
+    b = dev(syn.pack_codes(rng.integers(-8, 8, size=(n, k), dtype=np.int8)))
+    sa, sb = dev(rng.uniform(0.01, 0.5, size=(m, 1)).astype(np.float16)), dev(syn.weight_scales(n, 1, 1))
+    r = dev((rng.standard_normal((m, n)) * 2).astype(np.float16))
+    want = _ops.gemm_i4_dequant_add(a, b, sa, sb, r, 128)
+    assert same(ext.gemm_i4_dequant_add(a, b, sa, sb, r), want)
+    r2 = r.clone()
+    got = ext.gemm_i4_dequant_add(a, b, sa, sb, r2, 128, out=r2)         # in place on the residual stream
+    assert got.data_ptr() == r2.data_ptr() and same(r2, want)
+    assert same(ext.gemm_i4_dequant_add(a, b, sa, sb, r.view(3, 100, n), 128), want)
+    with pytest.raises(RuntimeError):
+        ext.gemm_i4_dequant_add(a, b, sa, sb, r[:, :32])
+    with pytest.raises(RuntimeError):
+        ext.gemm_i4_dequant_add(a, b, sa, sb, r.float())
+    gen = torch.Generator(device="cuda").manual_seed(4)
+    q = torch.randn(2, 150, 8, 128, device="cuda", generator=gen).half()
+    kc = torch.randn(2, 2, 200, 128, device="cuda", generator=gen).half()
+    vc = torch.randn(2, 2, 200, 128, device="cuda", generator=gen).half()
+    assert same(ext.prefill_attention(q, kc, vc, 50), _ops.prefill_attention(q, kc, vc, 50))
+    assert same(ext.prefill_attention(q, kc, vc, 0, scale=0.05), _ops.prefill_attention(q, kc, vc, 0, scale=0.05))
+    with pytest.raises(RuntimeError):
+        ext.prefill_attention(q, kc, vc, 51)                              # past + T exceeds the cache
+    with pytest.raises(RuntimeError):
+        ext.prefill_attention(q[..., :64].contiguous(), kc[..., :64].contiguous(), vc[..., :64].contiguous(), 0)
+    assert flh_amd._CUDA.prefill_attention is ext.prefill_attention
+
+
 def test_tensor_checks_raise_runtime_error(ext):
     a = torch.zeros(4, 64, dtype=torch.uint8, device="cuda")
     s = torch.ones(4, 1, dtype=torch.float16, device="cuda")
