@@ -833,6 +833,21 @@ def main():
     # calibration, not product: the vendor library's int8 GEMM (hipBLASLt through torch._int_mm: int8 operands,
     # int32 output, no nibble unpacking and no dequantisation) and fp16 GEMM on the same shapes, as a measure
     # of what fraction of the nominal matrix-core peak a tuned GEMM sustains on this device at these sizes
+    # Diagnostic, not product: the q / k / v-sized launch on operands of less switching activity.  The part is at its power
+    # limit under this kernel, and how fast it runs depends on how many operand bits toggle: all-zero codes show what the
+    # kernel's structure alone allows, a zero in every other code lies in between; codes quantised from normal data run
+    # within 2 % of uniform random ones.
+    activity = {}
+    n_act, k_act = 12288, 4096
+    sa_act = torch.full((M, 1), 0.01, dtype=torch.float16, device=dev)
+    sb_act = torch.full((n_act, 1), 0.01, dtype=torch.float16, device=dev)
+    for label, hi in (("uniform_random_codes", 256), ("every_other_code_zero", 16), ("all_zero_codes", 1)):
+        a_act = torch.randint(0, hi, (M, k_act // 2), dtype=torch.uint8, device=dev)
+        b_act = torch.randint(0, hi, (n_act, k_act // 2), dtype=torch.uint8, device=dev)
+        us = timed([lambda: ops.gemm_i4_dequant_o16(a_act, b_act, sa_act, sb_act)] * 20)
+        activity[label] = {"us": round(us, 2), "TOPS": round(gemm_ops(M, n_act, k_act) / (us * 1e-6) / 1e12, 1),
+                           "frac_of_peak": round(gemm_ops(M, n_act, k_act) / (us * 1e-6) / 1e12 / PEAK_INT8_TOPS, 4)}
+        del a_act, b_act
     vendor = None
     if not args.no_vendor_reference:
         vendor = {}
@@ -932,6 +947,7 @@ def main():
         f"llama3_8b_block_M={M},weight_groups_of_128": llama3,
         "llama3_8b_decode_linears,weight_groups_of_128": llama3_decode,
         "vendor_gemm_reference": vendor,
+        f"gemm_{n_act}x{k_act}_by_operand_activity": activity,
         "us_per_layer": round(ms_per_step * 1e3, 1),
         "shared_activation_launches": {"us_per_layer": round(ms_shared * 1e3, 1),
                                        "TOPS": round(sum(gemm_ops(M, n, k) for _, n, k, _ in LAYERS) / (ms_shared * 1e-3) / 1e12, 2),
