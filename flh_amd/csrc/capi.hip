@@ -2,6 +2,7 @@
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
+#include <mutex>
 
 #include "common.h"
 
@@ -20,6 +21,26 @@ int fail(int code, const char* fmt, ...) {
 int check_launch(const char* what) {
   const hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail(FLH_ELAUNCH, "%s: %s", what, hipGetErrorString(e));
+  return FLH_OK;
+}
+
+int current_device(int* dev, const char* what) {
+  if (hipGetDevice(dev) != hipSuccess) return fail(FLH_EDEVICE, "%s: no current HIP device", what);
+  if (*dev < 0 || *dev >= kMaxDevices)
+    return fail(FLH_EDEVICE, "%s: device index %d is beyond the %d this library keeps set-up for", what, *dev, kMaxDevices);
+  return FLH_OK;
+}
+
+int reserve_lds(const void* kernel, size_t bytes, LdsGrant& grant, const char* what) {
+  int dev = 0;
+  if (int rc = current_device(&dev, what)) return rc;
+  if (bytes <= grant.bytes[dev].load(std::memory_order_acquire)) return FLH_OK;
+  static std::mutex growing;                           // two sizes at once must not leave the smaller one in force
+  std::lock_guard<std::mutex> lock(growing);
+  if (bytes <= grant.bytes[dev].load(std::memory_order_relaxed)) return FLH_OK;
+  if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes) != hipSuccess)
+    return fail(FLH_ELAUNCH, "%s: cannot reserve %zu bytes of LDS", what, bytes);
+  grant.bytes[dev].store(bytes, std::memory_order_release);
   return FLH_OK;
 }
 

@@ -4,6 +4,8 @@
 #include <hip/hip_fp16.h>
 #include <stdint.h>
 
+#include <atomic>
+
 #include "../../include/flh_hip.h"
 
 namespace flh {
@@ -12,6 +14,18 @@ namespace flh {
 int fail(int code, const char* fmt, ...);
 // check for a launch error on the current device
 int check_launch(const char* what);
+
+// Set-up that a process repeats on every device it drives (a kernel's LDS reservation, a constant table, the address of
+// a __device__ array) is kept per device index.
+constexpr int kMaxDevices = 64;
+// the current device's index in [0, kMaxDevices) into *dev, or an error recorded for `what`
+int current_device(int* dev, const char* what);
+// the dynamic LDS a kernel has been granted on each device; one object with static storage (all zero) per kernel
+struct LdsGrant {
+  std::atomic<size_t> bytes[kMaxDevices];
+};
+// make `bytes` of dynamic LDS available to `kernel` on the current device unless that much already is
+int reserve_lds(const void* kernel, size_t bytes, LdsGrant& grant, const char* what);
 
 // true when any of the pointers is not a multiple of 16 bytes: rows are moved in 16-byte pieces (vector loads,
 // direct-to-LDS loads, vector stores), and every row is a whole number of such pieces from an aligned base only

@@ -330,13 +330,11 @@ constexpr size_t kScratchBytes = 16u << 20;            // 16 MiB: e.g. 31 sequen
 static __device__ __align__(256) unsigned char scratch[kScratchBytes];
 
 namespace {
-constexpr int kMaxDevices = 64;
 std::atomic<void*> g_scratch_ptr[kMaxDevices];         // per device: where that device's copy of `scratch` lives
 
 int scratch_of_current_device(void** out) {
   int dev = 0;
-  if (hipGetDevice(&dev) != hipSuccess) return fail(FLH_EDEVICE, "decode_attention: no current HIP device");
-  if (dev < 0 || dev >= kMaxDevices) return fail(FLH_EDEVICE, "decode_attention: device index %d out of range", dev);
+  if (int rc = current_device(&dev, "decode_attention")) return rc;
   void* ptr = g_scratch_ptr[dev].load(std::memory_order_acquire);
   if (!ptr) {
     const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));   // of the current device

@@ -587,17 +587,20 @@ __global__ __launch_bounds__(512) void rotate_quant_mfma_dense_kernel(const __ha
   if (!late) barrier_no_fence();
 }
 
-// The factor table of one size: built on first use (or by flh_init) on the legacy default stream and
-// waited for, so that later launches on any stream find it complete.  Not to be first reached under
-// stream capture -- call flh_init() before capturing.
+// The factor table of one size: built on first use on a device (or by flh_init with that device current) on the
+// legacy default stream and waited for, so that later launches on any stream find it complete.  Every device holds
+// its own copy of the array at its own address.  Not to be first reached under stream capture -- call flh_init()
+// before capturing.
 template <int DT>
 int dense_table(const h8** out) {
-  static std::atomic<const h8*> table{nullptr};
-  const h8* t = table.load(std::memory_order_acquire);
+  static std::atomic<const h8*> table[kMaxDevices];
+  int dev = 0;
+  if (int rc = current_device(&dev, "rotate_quant")) return rc;
+  const h8* t = table[dev].load(std::memory_order_acquire);
   if (!t) {
     static std::mutex once;
     std::lock_guard<std::mutex> lock(once);
-    t = table.load(std::memory_order_relaxed);
+    t = table[dev].load(std::memory_order_relaxed);
     if (!t) {
       constexpr int NFRAG = 2 * DT * DT;
       void* sym = nullptr;
@@ -607,7 +610,7 @@ int dense_table(const h8** out) {
       if (int rc = check_launch("build_dense_fragments")) return rc;
       if (hipStreamSynchronize(nullptr) != hipSuccess) return fail(FLH_ELAUNCH, "rotate_quant: building the factor table failed");
       t = (const h8*)sym;
-      table.store(t, std::memory_order_release);
+      table[dev].store(t, std::memory_order_release);
     }
   }
   *out = t;
@@ -623,12 +626,8 @@ int launch_dense_silu(const __half* gate, const __half* up, uint8_t* q, __half* 
   if (int rc = dense_table<DT>(&table)) return rc;
   const size_t smem = (size_t)NFRAG * 1024 + 64 + 2 * (size_t)DT * 4096;   // factor fragments, maxima, gate row, up row
   auto kern = rotate_quant_mfma_dense_kernel<DT, true, true>;
-  static std::atomic<bool> attr{false};
-  if (!attr.load(std::memory_order_acquire)) {
-    if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess)
-      return fail(FLH_ELAUNCH, "silu_mul_rotate_quant: cannot reserve %zu bytes of LDS", smem);
-    attr.store(true, std::memory_order_release);
-  }
+  static LdsGrant grant;
+  if (int rc = reserve_lds((const void*)kern, smem, grant, "silu_mul_rotate_quant")) return rc;
   hipLaunchKernelGGL(kern, dim3(M), dim3(512), smem, stream, gate, q, scales, table, M, 1.0f / sqrtf((float)K), 1.0f, up);
   return check_launch("silu_mul_rotate_quant");
 }
@@ -646,13 +645,8 @@ int launch_dense(const __half* x, uint8_t* q, __half* scales, uint32_t M, float 
   auto kern = f6 ? rotate_quant_mfma_dense_kernel<DT, false, false, true>
                  : split ? rotate_quant_mfma_dense_kernel<DT, true> : rotate_quant_mfma_dense_kernel<DT, false>;
   constexpr int kThreadsDense = 512;
-  static std::atomic<bool> attr[3] = {{false}, {false}, {false}};   // set-up is idempotent: a race only repeats it
-  const int variant = f6 ? 2 : split;
-  if (!attr[variant].load(std::memory_order_acquire)) {
-    if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess)
-      return fail(FLH_ELAUNCH, "rotate_quant: cannot reserve %zu bytes of LDS", smem);
-    attr[variant].store(true, std::memory_order_release);
-  }
+  static LdsGrant grants[3];                           // one per kernel variant
+  if (int rc = reserve_lds((const void*)kern, smem, grants[f6 ? 2 : split], "rotate_quant")) return rc;
   const unsigned blocks = split ? M : ((M + 3) / 4 < 256u ? (M + 3) / 4 : 256u);
   hipLaunchKernelGGL(kern, dim3(blocks), dim3(kThreadsDense), smem, stream, x, q, scales, table, M,
                      1.0f / sqrtf((float)K), clip, (const __half*)nullptr);

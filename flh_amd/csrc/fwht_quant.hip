@@ -963,13 +963,8 @@ extern "C" int flh_rotate_quant_i4(const flh_half* x, uint8_t* q_packed, flh_hal
   // the row in float32, a second copy for the dense factor's output and that factor's sign bits
   const size_t smem = (size_t)K * sizeof(float) * (Kd > 1 ? 2 : 1) + (Kd > 1 ? (((size_t)Kd * Kd + 7) / 8 / 16 + 2) * 16 : 0);   // + the byte after the last row's window
   if (smem > 160 * 1024 - 64) return fail(FLH_EINVAL, "rotate_quant: K = %u does not fit the LDS staging", K);
-  static std::atomic<size_t> reserved{0};             // largest LDS size granted so far (a race only repeats the call)
-  if (smem > reserved.load(std::memory_order_acquire)) {
-    if (hipFuncSetAttribute((const void*)rotate_quant_generic_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
-                            (int)smem) != hipSuccess)
-      return fail(FLH_ELAUNCH, "rotate_quant: cannot reserve %zu bytes of LDS", smem);
-    reserved.store(smem, std::memory_order_release);
-  }
+  static LdsGrant grant;                               // grows to the largest row asked for
+  if (int rc = reserve_lds((const void*)rotate_quant_generic_kernel, smem, grant, "rotate_quant")) return rc;
   hipLaunchKernelGGL(rotate_quant_generic_kernel, dim3(M), dim3(kGenericThreads), smem, st, xh, q_packed, sh, yh, K,
                      hadamard == FLH_HAD_NONE ? 0 : P, Kd, norm, scale_group, clip_ratio);
   return check_launch("rotate_quant_generic");

@@ -680,12 +680,8 @@ int launch(GemmArgs a, hipStream_t stream) {
   const size_t smem = (size_t)KS * STAGES * (BM + BN) * kStageBytes +
                       (EPI == kRowScale ? (BM + BN) * 2 : (EPI == kGroupScale || EPI == kTokenGroup) ? (BM + BN) * 32 : 0);
   auto kern = gemm_i4_kernel<BM, BN, WM, WN, STAGES, EPI, GROUP, KS, SWIGLU, ROPE>;
-  static std::atomic<bool> attr_set{false};   // set-up is idempotent: a race only repeats it  // per instantiation
-  if (!attr_set.load(std::memory_order_acquire)) {
-    if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess)
-      return fail(FLH_ELAUNCH, "gemm: cannot reserve %zu bytes of LDS", smem);
-    attr_set.store(true, std::memory_order_release);
-  }
+  static LdsGrant grant;                               // per instantiation
+  if (int rc = reserve_lds((const void*)kern, smem, grant, "gemm")) return rc;
   hipLaunchKernelGGL(kern, dim3(a.tiles_m * a.tiles_n), dim3(64 * (BM / WM) * (BN / WN) * KS), smem, stream, a);
   return check_launch("gemm_i4");
 }

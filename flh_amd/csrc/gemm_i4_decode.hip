@@ -189,13 +189,9 @@ int launch_decode(const GemmArgs& a, hipStream_t stream) {
   const size_t smem = EPI == kGroupScale ? (size_t)KT * MT * 1024 + (size_t)KT * 128 : (size_t)kWaves * MT * 1024;
   auto kern = gemm_i4_decode_kernel<MT, EPI>;
   if constexpr (EPI == kGroupScale) {
-    static std::atomic<bool> attr_set{false};   // set-up is idempotent: a race only repeats it
-    if (!attr_set.load(std::memory_order_acquire)) {
-      const int cap = kGroupMaxKT * MT * 1024 + kGroupMaxKT * 128;
-      if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, cap) != hipSuccess)
-        return fail(FLH_ELAUNCH, "gemm (decode): cannot reserve %d bytes of LDS", cap);
-      attr_set.store(true, std::memory_order_release);
-    }
+    static LdsGrant grant;                             // per instantiation; sized for the longest rows it takes
+    if (int rc = reserve_lds((const void*)kern, (size_t)kGroupMaxKT * MT * 1024 + (size_t)kGroupMaxKT * 128, grant, "gemm (decode)"))
+      return rc;
   }
   GemmArgs g = a;
   const int blocks = decode_blocks(g);

@@ -276,13 +276,8 @@ extern "C" int flh_prefill_attention_f16(const flh_half* q, const flh_half* k_ca
   if (!(scale > 0.f)) return fail(FLH_EINVAL, "prefill_attention: the scale must be positive");
   const size_t smem = 4 * (size_t)kTileBytes;          // 64 KiB: two workgroups per compute unit
   static_assert(4 * 32 * kOutPitch <= 4 * kTileBytes, "the output staging tiles reuse the K / V buffers");
-  static std::atomic<bool> attr_set{false};            // set-up is idempotent: a race only repeats it
-  if (!attr_set.load(std::memory_order_acquire)) {
-    if (hipFuncSetAttribute((const void*)prefill_attention_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) !=
-        hipSuccess)
-      return fail(FLH_ELAUNCH, "prefill_attention: cannot reserve %zu bytes of LDS", smem);
-    attr_set.store(true, std::memory_order_release);
-  }
+  static LdsGrant grant;
+  if (int rc = reserve_lds((const void*)prefill_attention_kernel, smem, grant, "prefill_attention")) return rc;
   const unsigned blocks = (T + kQueriesPerBlock - 1) / kQueriesPerBlock;
   hipLaunchKernelGGL(prefill_attention_kernel, dim3(blocks * Hq * B), dim3(256), smem, (hipStream_t)stream, (const __half*)q,
                      (const __half*)k_cache, (const __half*)v_cache, (__half*)out, (int)T, (int)Hq, (int)Hkv, (int)past,

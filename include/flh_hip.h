@@ -36,9 +36,9 @@ typedef uint16_t flh_half; /* IEEE binary16 bit pattern */
 int flh_abi_version(void);
 /* message of the last failing call on this thread ("" if none) */
 const char* flh_last_error(void);
-/* one-time set-up: checks the device and builds the constant tables of the matrix-core rotation (a short
- * kernel on the default stream, waited for).  Optional -- first use does the same -- but call it before
- * capturing a stream into a graph, since that first use synchronises. */
+/* set-up of the current device, once per device: checks the device and builds the constant tables of the
+ * matrix-core rotation (a short kernel on the default stream, waited for).  Optional -- first use on a device does
+ * the same -- but call it before capturing a stream into a graph, since that first use synchronises. */
 int flh_init(void);
 
 /* ---------------------------------------------------------------------------------
