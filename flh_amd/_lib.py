@@ -83,6 +83,7 @@ _SIG = {
     "flh_rotate_quant_f6": (_c.c_int, [_PTR, _PTR, _PTR, _c.c_int, _PTR, _c.c_float, _PTR, _PTR, _c.c_uint32, _c.c_uint32,
                                       _c.c_int, _c.c_float, _PTR]),
     "flh_silu_mul_f16": (_c.c_int, [_PTR, _PTR, _PTR, _c.c_uint64, _PTR]),
+    "flh_add_rmsnorm_f16": (_c.c_int, [_PTR, _PTR, _PTR, _c.c_float, _PTR, _PTR, _c.c_uint32, _c.c_uint32, _PTR]),
     "flh_silu_mul_rotate_quant_i4": (_c.c_int, [_PTR, _PTR, _PTR, _PTR, _c.c_uint32, _c.c_uint32, _PTR]),
     "flh_fwht_f16_inplace": (_c.c_int, [_PTR, _c.c_uint32, _c.c_int, _PTR]),
     "flh_rotate_quant_i4": (_c.c_int, [_PTR, _PTR, _PTR, _PTR, _c.c_uint32, _c.c_uint32, _c.c_int, _c.c_int,

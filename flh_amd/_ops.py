@@ -751,6 +751,31 @@ def silu_mul(gate, up):
     return out
 
 
+def add_rmsnorm(x, weight=None, eps=1e-5, add=None, return_sum=False):
+    """RMSNorm on its own, in one launch, optionally behind the residual addition: x [..., K] fp16 (`add` of the same
+    shape or None; the row is then fp16(x + add)), weight [K] fp16 or None -> fp16 tensor of x's shape, statistics in
+    float32 (flh/nn/normalization.py:12-20); with return_sum also the stored sum x + add, first."""
+    _check(x.is_cuda and x.dtype == torch.float16 and x.dim() >= 1 and x.is_contiguous(),
+           "Input tensor must be a contiguous float16 CUDA tensor")
+    K = x.size(-1)
+    _check(K % 8 == 0 and 0 < K <= 16384, "Last dimension must be a multiple of 8, at most 16384")
+    if add is not None:
+        _check(add.is_cuda and add.dtype == torch.float16 and add.shape == x.shape and add.is_contiguous()
+               and add.device == x.device, "add must be a contiguous float16 CUDA tensor of x's shape")
+    _check(not return_sum or add is not None, "return_sum needs add")
+    if weight is not None:
+        _check(weight.is_cuda and weight.dtype == torch.float16 and weight.is_contiguous() and weight.numel() == K
+               and weight.device == x.device, "weight must be a contiguous float16 CUDA tensor of K values")
+    out = torch.empty_like(x)
+    total = torch.empty_like(x) if return_sum else None
+    M = x.numel() // K
+    if M:
+        _run("flh_add_rmsnorm_f16", x.device, x.data_ptr(), add.data_ptr() if add is not None else None,
+             weight.data_ptr() if weight is not None else None, float(eps), out.data_ptr(),
+             total.data_ptr() if total is not None else None, M, K, _stream(x))
+    return (total, out) if return_sum else out
+
+
 def silu_mul_rotate_and_quantize_i4(gate, up):
     """Decode-sized batches: rotate_and_quantize_i4(silu(gate) * up, hadamard="fast") in one launch that never stores the
     product: gate, up [M, K] fp16 with K = 11008 or 14336, M <= 256 -> (q [M, K/2] u8, scales [M, 1] fp16)."""

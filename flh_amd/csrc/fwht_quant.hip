@@ -311,6 +311,59 @@ __global__ __launch_bounds__(256) void rmsnorm_group_kernel(const __half* __rest
   }
 }
 
+// RMSNorm on its own (a model's final norm, in front of an fp16 head), optionally behind the residual addition: one
+// workgroup per row of K = 8 * chunks values (K <= 16384), the statistics and roundings of rmsnorm_group_kernel;
+// with `add` the row is fp16(x + add), one rounding per value, stored to sum_out as well when that is given.
+__global__ __launch_bounds__(256) void add_rmsnorm_kernel(const __half* __restrict__ x, const __half* __restrict__ add,
+                                                          const __half* __restrict__ weight, __half* __restrict__ out,
+                                                          __half* __restrict__ sum_out, uint32_t K, float eps) {
+  constexpr int MAXC = 8;
+  __shared__ float part[4];
+  const int tid = threadIdx.x;
+  const uint32_t chunks = K / 8;
+  const size_t row = (size_t)blockIdx.x * K;
+  h8 raw[MAXC];
+  float ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < MAXC; ++i) {
+    const uint32_t c = tid + 256u * i;
+    if (c < chunks) {
+      raw[i] = *(const h8*)(x + row + (size_t)c * 8);
+      if (add) {
+        raw[i] = __builtin_bit_cast(h8, add_h8(__builtin_bit_cast(v4i, raw[i]), *(const v4i*)(add + row + (size_t)c * 8)));
+        if (sum_out) *(h8*)(sum_out + row + (size_t)c * 8) = raw[i];
+      }
+#pragma unroll
+      for (int e = 0; e < 8; ++e) ss = __builtin_fmaf((float)raw[i][e], (float)raw[i][e], ss);
+    }
+  }
+  ss += dpp_f<kDppQuadXor1>(ss);
+  ss += dpp_f<kDppQuadXor2>(ss);
+  ss += dpp_f<kDppRowHalfMirror>(ss);
+  ss += dpp_f<kDppRowMirror>(ss);
+  ss += lane_xor_f<16>(ss);
+  ss += lane_xor_f<32>(ss);
+  if ((tid & 63) == 0) part[tid >> 6] = ss;
+  __syncthreads();
+  const float total = (part[0] + part[1]) + (part[2] + part[3]);
+  const float inv = 1.0f / __builtin_sqrtf(total / (float)K + eps);
+#pragma unroll
+  for (int i = 0; i < MAXC; ++i) {
+    const uint32_t c = tid + 256u * i;
+    if (c < chunks) {
+      h8 w8, y;
+      if (weight) w8 = *(const h8*)(weight + (size_t)c * 8);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        float t = round_here((float)raw[i][e] * inv);
+        if (weight) t = round_here(t * (float)w8[e]);
+        y[e] = (_Float16)t;
+      }
+      *(h8*)(out + row + (size_t)c * 8) = y;
+    }
+  }
+}
+
 // ------------------------------------------------------------------------------------
 // 2. wave-per-row kernel, float32 butterflies, K = 512 * J: four rows per workgroup, rotate_quant_row (rotate_row.h)
 // ------------------------------------------------------------------------------------
@@ -868,6 +921,19 @@ extern "C" int flh_silu_mul_f16(const flh_half* gate, const flh_half* up, flh_ha
   hipLaunchKernelGGL(silu_mul_kernel, dim3((unsigned)((n / 8 + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
                      (const __half*)gate, (const __half*)up, (__half*)out, n / 8);
   return check_launch("silu_mul_kernel");
+}
+
+extern "C" int flh_add_rmsnorm_f16(const flh_half* x, const flh_half* add, const flh_half* weight, float eps, flh_half* out,
+                                   flh_half* sum_out, uint32_t M, uint32_t K, void* stream) {
+  if (!x || !out) return fail(FLH_EINVAL, "add_rmsnorm: null pointer");
+  if (sum_out && !add) return fail(FLH_EINVAL, "add_rmsnorm: sum_out is the stored sum x + add and needs add");
+  if (misaligned16(x, add, weight, out, sum_out)) return fail(FLH_EINVAL, "add_rmsnorm: tensors must be 16-byte aligned");
+  if (K == 0 || K % 8 || K > 16384) return fail(FLH_EINVAL, "add_rmsnorm: K (%u) must be a multiple of 8, at most 16384", K);
+  if (!(eps >= 0.f)) return fail(FLH_EINVAL, "add_rmsnorm: eps must not be negative");
+  if (M == 0) return FLH_OK;
+  hipLaunchKernelGGL(add_rmsnorm_kernel, dim3(M), dim3(256), 0, (hipStream_t)stream, (const __half*)x, (const __half*)add,
+                     (const __half*)weight, (__half*)out, (__half*)sum_out, K, eps);
+  return check_launch("add_rmsnorm_kernel");
 }
 
 extern "C" int flh_silu_mul_rotate_quant_i4(const flh_half* gate, const flh_half* up, uint8_t* q_packed, flh_half* scales,

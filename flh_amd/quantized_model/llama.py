@@ -3,8 +3,9 @@ decode step that runs from a preallocated key / value cache and can be captured 
 
 Data flow of the reference's FLH_LlamaForCausalLM.forward (flh/quantized_model/modeling_llama.py:668-693:
 embedding -> [group configuration only: Hadamard of every 128 channels of the embeddings] -> decoder layers ->
-final RMSNorm -> lm_head), with the layers of decoder_layer.py.  The int4 linears are this library's kernels; the
-embedding, RoPE, attention, norms outside the fused launches and the head are stock torch ops, as in the reference.
+final RMSNorm -> lm_head), with the layers of decoder_layer.py.  The int4 linears, the rotary embedding, attention and
+the norms (the final one with the last residual addition in its launch) are this library's kernels on the fused path;
+the embedding and the head are stock torch ops, as in the reference.
 Weights are random (there are no checkpoints here): `random_init` draws fp16 weights layer by layer on the device and
 quantises them through the same kernels a loader would use.
 """
@@ -58,7 +59,8 @@ def reference_key(key):
 class W4A4LlamaModel(torch.nn.Module):
     def __init__(self, shape, activation="token", weight_group_size=128, fused=True, device="cpu"):
         super().__init__()
-        self.shape, self.activation = shape, activation
+        self.shape, self.activation, self.fused = shape, activation, fused
+        self._norm16 = None                 # (version key, fp16 copy) of the final norm's weight
         self.embed_tokens = torch.nn.Embedding(shape.vocab_size, shape.hidden_size, device=device, dtype=torch.float16)
         self.layers = torch.nn.ModuleList(
             W4A4DecoderLayer(shape.hidden_size, shape.num_heads, shape.num_kv_heads, shape.intermediate_size, shape.eps,
@@ -241,10 +243,21 @@ class W4A4LlamaModel(torch.nn.Module):
         for i, layer in enumerate(self.layers):
             x, pending, _ = layer.forward_deferred(x, pending, cos, sin, cache.layer(i) if cache is not None else None,
                                                    positions)
-        if pending is not None:
-            x = x + pending
-        x = self.norm(x)
+        x = self._final_norm(x, pending)
         return x if return_hidden else self.lm_head(x)
+
+    def _final_norm(self, x, pending):
+        """The last residual addition and the final RMSNorm: one launch on the fused path (the roundings of the two
+        torch expressions: fp16 sum, float32 statistics, two float32 products, fp16), torch's ten otherwise."""
+        w = self.norm.weight
+        if not (self.fused and x.is_cuda and x.dtype == torch.float16 and x.size(-1) % 8 == 0 and x.size(-1) <= 16384):
+            return self.norm(x if pending is None else x + pending)
+        key = (w.data_ptr(), w._version)
+        if self._norm16 is None or self._norm16[0] != key:
+            self._norm16 = (key, w.detach().to(torch.float16).contiguous())
+        import flh_amd
+        return flh_amd._CUDA.add_rmsnorm(x.contiguous(), self._norm16[1], self.norm.eps,
+                                         add=None if pending is None else pending.contiguous())
 
     def capture_decode_step(self, batch, kv_len, cache=None, with_head=True):
         """Record one decode step (batch x 1 token, attention over `kv_len` cached positions, the new token in slot

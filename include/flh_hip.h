@@ -314,6 +314,14 @@ int flh_add_rmsnorm_rotate_quant_i4(const flh_half* x, const flh_half* add, flh_
 int flh_silu_mul_rotate_quant_i4(const flh_half* gate, const flh_half* up, uint8_t* q_packed, flh_half* scales,
                                  uint32_t M, uint32_t K, void* stream);
 
+/* RMSNorm on its own, optionally behind the residual addition -- a model's final norm in front of its fp16 head
+ * (flh/nn/normalization.py:12-20 after the last residual addition of flh/quantized_model/modeling_llama.py:600-618):
+ * s = add ? fp16(x + add) : x;  out = fp16( fl32(fl32(s) * rsqrt(sum(s^2) / K + eps)) * fl32(weight) ), statistics in
+ * float32.  x, add (or NULL), out, sum_out (or NULL; receives s, needs add) [M, K] fp16; weight [K] fp16 or NULL (ones);
+ * K a multiple of 8, at most 16384.  One launch for torch's addition and the eight kernels of the norm's expression. */
+int flh_add_rmsnorm_f16(const flh_half* x, const flh_half* add, const flh_half* weight, float eps, flh_half* out,
+                        flh_half* sum_out, uint32_t M, uint32_t K, void* stream);
+
 /* The same product on its own: out[i] = fp16(fp16(silu(gate[i])) * up[i]) for n fp16 values (n a multiple of 8; out may
  * be gate or up).  One launch for the two torch kernels of modeling_llama.py:522-526 where no quantiser follows directly. */
 int flh_silu_mul_f16(const flh_half* gate, const flh_half* up, flh_half* out, uint64_t n, void* stream);

@@ -251,3 +251,61 @@ def test_residual_add_argument_errors(ops):
         ops.add_rmsnorm_rotate_and_quantize_i4(x[:, :768].contiguous(), x[:, :768].contiguous(), None, 1e-5)
     with pytest.raises(RuntimeError):
         ops.add_rmsnorm_rotate_and_quantize_i4(x, x.float(), None, 1e-5)
+
+
+# ---- RMSNorm on its own (a model's final norm), optionally behind the residual addition ---------------------------------
+
+VALUE_RATE = 1e-3    # fraction of fp16 outputs allowed to differ from the CPU evaluation (by one ulp: summation order)
+
+
+@pytest.mark.parametrize("m,k", [(1, 4096), (16, 4096), (5, 5120), (3, 8192), (7, 16384), (9, 264), (33, 8)])
+@pytest.mark.parametrize("weighted", [False, True])
+@pytest.mark.parametrize("with_add", [False, True])
+def test_add_rmsnorm(ops, m, k, weighted, with_add):
+    from oracle import prologue as P
+    rng = np.random.default_rng(m + k + weighted + 2 * with_add)
+    x = (rng.standard_normal((m, k)) * rng.uniform(0.05, 30, (m, 1))).astype(np.float16)
+    a = (rng.standard_normal((m, k)) * rng.uniform(0.05, 30, (m, 1))).astype(np.float16) if with_add else None
+    w = rng.uniform(0.3, 2.5, k).astype(np.float16) if weighted else None
+    print(f"case add_rmsnorm m={m} k={k} weighted={weighted} add={with_add}", flush=True)
+    if with_add:
+        total, y = ops.add_rmsnorm(dev(x), dev(w) if weighted else None, 1e-5, add=dev(a), return_sum=True)
+        s = (x.astype(np.float32) + a.astype(np.float32)).astype(np.float16)      # one rounding per value
+        assert np.array_equal(host(total).view(np.uint16), s.view(np.uint16))
+        assert np.array_equal(host(ops.add_rmsnorm(dev(x), dev(w) if weighted else None, 1e-5, add=dev(a))).view(np.uint16),
+                              host(y).view(np.uint16))
+    else:
+        s, y = x, ops.add_rmsnorm(dev(x), dev(w) if weighted else None, 1e-5)
+    ref = P.rmsnorm_f16(s, w, 1e-5)
+    d = np.abs(host(y).view(np.int16).astype(np.int32) - ref.view(np.int16).astype(np.int32))
+    assert d.max() <= 1 and np.mean(d != 0) <= VALUE_RATE, (d.max(), np.mean(d != 0))
+
+
+@pytest.mark.parametrize("k", [8, 4096, 16384])
+def test_add_rmsnorm_exact_data_bit_exact(ops, k):
+    """Rows of +-1 with eps = 0 (as the sum of +-3 and -+2): the mean square is exactly 1 and every output is
+    sign * weight bit for bit; a row of zeros with eps > 0 stays zero."""
+    rng = np.random.default_rng(k)
+    sign = rng.choice([-1.0, 1.0], size=(11, k)).astype(np.float16)
+    w = rng.uniform(0.3, 2.5, k).astype(np.float16)
+    y = ops.add_rmsnorm(dev(sign * np.float16(3)), dev(w), 0.0, add=dev(sign * np.float16(-2)))
+    assert np.array_equal(host(y).view(np.uint16), (sign * w).astype(np.float16).view(np.uint16))
+    z = ops.add_rmsnorm(torch.zeros(2, k, dtype=torch.float16, device="cuda"), dev(w), 1e-5)
+    assert not host(z).any()
+
+
+def test_add_rmsnorm_argument_errors(ops):
+    x = torch.zeros(4, 4096, dtype=torch.float16, device="cuda")
+    for bad in (lambda: ops.add_rmsnorm(x, None, 1e-5, add=x[:2]),
+                lambda: ops.add_rmsnorm(x[:, :4092].contiguous()),
+                lambda: ops.add_rmsnorm(torch.zeros(2, 16392, dtype=torch.float16, device="cuda")),
+                lambda: ops.add_rmsnorm(x.float()),
+                lambda: ops.add_rmsnorm(x, x[0, :100].contiguous()),
+                lambda: ops.add_rmsnorm(x, None, 1e-5, return_sum=True)):
+        with pytest.raises(RuntimeError):
+            bad()
+    from flh_amd import _lib
+    lib = _lib.load()
+    assert lib.flh_add_rmsnorm_f16(x.data_ptr(), None, None, 1e-5, x.data_ptr(), x.data_ptr(), 4, 4096, None) != 0   # sum_out without add
+    assert b"sum_out" in lib.flh_last_error()
+    assert ops.add_rmsnorm(x[:0]).shape == (0, 4096)
