@@ -93,6 +93,80 @@ def cpu_baseline(m_sample, min_seconds=10.0, budget_s=30.0):
                       "(numpy oracle, float32 BLAS matmul of unpacked codes)"}
 
 
+def operand_activity(torch, ops, m, launches, smi):
+    """The q / k / v-sized launch (m x 12288 x 4096, one scale per row) on operands of decreasing switching activity:
+    what separates the power limit of the part from the structure of the kernel.  Per case: median HIP-event time of
+    `launches` back-to-back launches, and -- from a second thread, while the same launch keeps running -- the engine
+    clock and the socket power rocm-smi reports.  A counter run (rocprofv3 --pmc GRBM_GUI_ACTIVE
+    SQ_VALU_MFMA_BUSY_CYCLES SQ_BUSY_CU_CYCLES) of this mode sees `launches` dispatches per case, in the order of the
+    cases, behind the warm-up dispatches."""
+    import re
+    import subprocess
+    import threading
+    dev = torch.device("cuda:0")
+    n, k = 12288, 4096
+    sa = torch.full((m, 1), 0.01, dtype=torch.float16, device=dev)
+    sb = torch.full((n, 1), 0.01, dtype=torch.float16, device=dev)
+    out = {"shape": f"{m}x{n}x{k}", "launches_per_case": launches, "cases": {}}
+
+    def smi_reading():
+        try:
+            txt = subprocess.run(["rocm-smi", "--showclocks", "--showpower"], capture_output=True, text=True, timeout=30).stdout
+        except Exception:  # noqa: BLE001 -- the reading is optional
+            return None, None
+        mc = re.search(r"sclk clock level: \d+: \((\d+)Mhz\)", txt)
+        mp = re.search(r"Power \(W\): ([0-9.]+)", txt)
+        watts = float(mp.group(1)) if mp else None
+        if watts is None:                                 # the tool prints no power on some boxes: the driver's own file
+            import glob
+            for f in glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*/power1_average") + \
+                    glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*/power1_input"):
+                try:
+                    watts = int(open(f).read().strip()) / 1e6
+                    break
+                except Exception:  # noqa: BLE001
+                    pass
+        return (int(mc.group(1)) if mc else None), watts
+
+    for label, hi in (("uniform_random_codes", 256), ("every_other_code_zero", 16), ("all_zero_codes", 1)):
+        a = torch.randint(0, hi, (m, k // 2), dtype=torch.uint8, device=dev)
+        b = torch.randint(0, hi, (n, k // 2), dtype=torch.uint8, device=dev)
+        for _ in range(300):                              # steady clocks for this data
+            ops.gemm_i4_dequant_o16(a, b, sa, sb)
+        torch.cuda.synchronize()
+        pairs = []
+        for _ in range(launches):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            ops.gemm_i4_dequant_o16(a, b, sa, sb)
+            e1.record()
+            pairs.append((e0, e1))
+        torch.cuda.synchronize()
+        us = float(np.median([x.elapsed_time(y) * 1e3 for x, y in pairs]))
+        case = {"us": round(us, 2), "TOPS": round(gemm_ops(m, n, k) / (us * 1e-6) / 1e12, 1),
+                "frac_of_peak": round(gemm_ops(m, n, k) / (us * 1e-6) / 1e12 / PEAK_INT8_TOPS, 4)}
+        if smi:
+            reading = [None, None]
+
+            def sample():
+                time.sleep(0.7)
+                reading[0], reading[1] = smi_reading()
+            th = threading.Thread(target=sample)
+            th.start()
+            t0 = time.perf_counter()
+            while th.is_alive() and time.perf_counter() - t0 < 20.0:
+                for _ in range(100):
+                    ops.gemm_i4_dequant_o16(a, b, sa, sb)
+                torch.cuda.synchronize()
+            th.join()
+            case["engine_MHz"], case["socket_W"] = reading
+            if reading[0]:
+                case["frac_of_peak_at_that_clock"] = round(case["frac_of_peak"] * 2400.0 / reading[0], 4)
+        out["cases"][label] = case
+        del a, b
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -112,6 +186,12 @@ def main():
     ap.add_argument("--launches", choices=["layer", "seven"], default="layer",
                     help="GEMM launches of the timed step: the four a decoder layer issues (q/k/v in one launch, gate and "
                          "up in one launch that stores silu(gate)*up), or one per linear; the other form is reported beside it")
+    ap.add_argument("--operand-activity-only", type=int, default=0, metavar="LAUNCHES",
+                    help="diagnostic mode: only the q/k/v-sized GEMM launch (2048 x 12288 x 4096) on uniform random codes, "
+                         "on codes with every other one zero and on all-zero codes, LAUNCHES back-to-back launches each "
+                         "(in that order; the run under rocprofv3 --pmc that profiles/ summarises reads its counters per "
+                         "dispatch), with the engine clock and socket power rocm-smi reports during each case")
+    ap.add_argument("--no-smi", action="store_true", help="with --operand-activity-only: do not start rocm-smi")
     ap.add_argument("--large-tokens", type=int, default=16384,
                     help="token count of the extra Hadamard-quant launches that amortise the launch floor")
     args = ap.parse_args()
@@ -126,6 +206,9 @@ def main():
     if not torch.cuda.is_available():
         sys.exit("bench.py needs the MI355X (no CPU fallback for the product path)")
     M = args.tokens
+    if args.operand_activity_only:
+        print(json.dumps(operand_activity(torch, ops, M, args.operand_activity_only, not args.no_smi)))
+        return
     acts_h, weights_h = make_inputs(M)
     dev = torch.device("cuda:0")
     acts = {k: torch.from_numpy(v).to(dev) for k, v in acts_h.items()}

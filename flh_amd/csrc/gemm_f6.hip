@@ -75,7 +75,7 @@ void gemm_f6_kernel(const GemmArgs p) {
   constexpr bool GROUPED = EPI == kGroupScale || EPI == kTokenGroup;
   constexpr bool token_scale = EPI == kTokenGroup;
   constexpr int SCROWS = BM + BN;
-  static_assert(!GROUPED || (SCROWS <= T && STAGES == 3), "one thread per scale row; prefetch relies on the full wait");
+  static_assert(!GROUPED || SCROWS <= T, "one thread per scale row");
 
   extern __shared__ __align__(1024) uint8_t lds[];    // [STAGES][STAGE], then the tile's scales
 
@@ -125,7 +125,7 @@ void gemm_f6_kernel(const GemmArgs p) {
     src_of[i] = isA ? 0 : second ? 2 : 1;
   }
   const int KT = p.K / 128;
-  auto issue_stage = [&](int stage, int kt) {
+  auto issue_stage = [&](int stage, int kt) __attribute__((always_inline)) {
     const int k = kt < KT ? kt : KT - 1;              // past the end: harmless reload, keeps the wait counts fixed
     const unsigned base = lds0 + stage * STAGE + first_i * 1024;
     const uint8_t* ka = p.A + (size_t)k * p.M * kBlockBytes;   // slab k of either operand
@@ -159,25 +159,46 @@ void gemm_f6_kernel(const GemmArgs p) {
   const int sw = (frag_row >> 3) & 1;
   // byte offsets inside a tile row of the three chunks of this wave half
   const int c0 = ((3 * frag_chunk) ^ sw) * 16, c1 = ((3 * frag_chunk + 1) ^ sw) * 16, c2 = ((3 * frag_chunk + 2) ^ sw) * 16;
+  // (the second half of the middle chunk gets an offset of its own that the compiler cannot see through: adjacent
+  // 8-byte reads would be merged into one 16-byte read again and taken apart with copy instructions)
+  int c1b = c1 + 8;
+  asm("" : "+v"(c1b));
   const int a_base = (wm + frag_row) * kBlockBytes, b_base = (BM + wn + frag_row) * kBlockBytes;
 
   constexpr int NF = TM + TN;                          // fragments per stage (A first, then B)
-  v4i fr[2][NF][3];                                    // [parity][fragment][chunk]: 48 bytes = the operands of two MFMAs
-  auto read_stage = [&](int par, int stage) {
-    const uint8_t* st = lds + stage * STAGE;
+  // The 48 bytes a lane reads of a row are the operands of two MFMAs, 24 bytes (six registers) each.  They are read as
+  // 16 + 8 and 8 + 16 bytes, so that every piece lands in the registers of the operand it belongs to and no copy
+  // instruction is needed to assemble an operand (a 16-byte read of the middle chunk would straddle the two).
+  v4i fa[2][NF], fd[2][NF];                            // [parity][fragment]: bytes 0-15 and 32-47 of the lane's 48
+  v2i fb[2][NF], fc[2][NF];                            // ... bytes 16-23 and 24-31
+  // All fragments of a stage are read one stage ahead of the MFMAs that use them.
+  // byte offset of fragment f's row inside a stage: every fragment gets an offset register of its own that the compiler
+  // cannot see through, or it would merge
+  // the 8-byte reads of two fragments (3072 bytes apart) into one instruction with four result registers and take
+  // them apart again with copy instructions.
+  int frag_off[NF];
 #pragma unroll
-    for (int f = 0; f < NF; ++f) {
-      const uint8_t* row = st + (f < TM ? a_base + f * 32 * kBlockBytes : b_base + (f - TM) * 32 * kBlockBytes);
-      fr[par][f][0] = *(const v4i*)(row + c0);
-      fr[par][f][1] = *(const v4i*)(row + c1);
-      fr[par][f][2] = *(const v4i*)(row + c2);
-    }
+  for (int f = 0; f < NF; ++f) {
+    frag_off[f] = f < TM ? a_base + f * 32 * kBlockBytes : b_base + (f - TM) * 32 * kBlockBytes;
+    if (f != 0 && f != TM) asm("" : "+v"(frag_off[f]));
+  }
+  auto read_frag = [&](auto par_tag, auto f_tag, int stage) __attribute__((always_inline)) {
+    constexpr int par = decltype(par_tag)::value, f = decltype(f_tag)::value;
+    const uint8_t* row = lds + stage * STAGE + frag_off[f];
+    fa[par][f] = *(const v4i*)(row + c0);
+    fb[par][f] = *(const v2i*)(row + c1);
+    fc[par][f] = *(const v2i*)(row + c1b);
+    fd[par][f] = *(const v4i*)(row + c2);
+  };
+  auto read_stage = [&](auto par_tag, int stage) __attribute__((always_inline)) {
+    static_for<NF>([&](auto f_tag) { read_frag(par_tag, f_tag, stage); });
   };
   auto operand = [&](int par, int f, int m) {
-    const v4i a = fr[par][f][0], b = fr[par][f][1], c = fr[par][f][2];
-    return m == 0 ? v8i{a[0], a[1], a[2], a[3], b[0], b[1], 0, 0} : v8i{b[2], b[3], c[0], c[1], c[2], c[3], 0, 0};
+    const v4i a = fa[par][f], d = fd[par][f];
+    const v2i b = fb[par][f], c = fc[par][f];
+    return m == 0 ? v8i{a[0], a[1], a[2], a[3], b[0], b[1], 0, 0} : v8i{c[0], c[1], d[0], d[1], d[2], d[3], 0, 0};
   };
-  auto mfma_stage = [&](int par) {
+  auto mfma_stage = [&](int par) __attribute__((always_inline)) {
 #pragma unroll
     for (int m = 0; m < 2; ++m)
 #pragma unroll
@@ -188,67 +209,142 @@ void gemm_f6_kernel(const GemmArgs p) {
                                                                      acc[i][j], kBf6, kBf6, 0, 0, 0, 0);
   };
 
-  // ---- group scales travel through LDS (as in the int8 kernel): thread t owns row t of the tile's BM activation
-  // rows and BN weight rows, fetches that row's next eight group scales one block ahead and stores them
-  // transposed, sc[buffer][group & 7][row], where the fold reads four channels' scales as one 8-byte run
-  __half* const sc = (__half*)(lds + STAGES * STAGE);  // [2][8][SCROWS]
-  unsigned short sraw[8];
-  const bool sc_thread = tid < SCROWS;
-  const int sc_cols = tid < BM ? p.a_cols : p.b_cols;
-  const int sc_brow = min(tid, SCROWS - 1) - BM;      // weight row of the tile this thread fetches scales for
+  // ---- group scales travel through LDS, eight groups (= eight K steps) at a time.  Thread t owns row t of the tile's
+  // BM activation rows and BN weight rows (with one scale per token: of the BN weight rows only).  In the first step of
+  // a block of eight it requests the row's eight scales of the NEXT block -- one 16-byte load where rows of scales are
+  // dword-aligned runs of at least eight, else eight clamped 2-byte loads -- and in the block's second step, behind
+  // that step's full wait and barrier, it stores them transposed into scl[block & 1][group - first][row], where a step
+  // reads a lane's channel scale as one 2-byte piece and four tokens' scales as one 8-byte run.  (One 2-byte request
+  // per row and group costs as many cache-line requests as the operands themselves.)  The two steps with this extra
+  // work are code of their own; the other steps of a block stay free of branches, which the interleaving of matrix
+  // and vector work below depends on.
+  constexpr int SCR = token_scale ? BN : SCROWS;       // rows of scales kept
+  constexpr int SCR0 = token_scale ? BM : 0;           // first tile row that has any
+  __half* const scl = (__half*)(lds + STAGES * STAGE); // [2][8][SCR]
+  const int sc_row = min(tid, SCROWS - 1);             // (threads past the last row repeat it)
+  const bool sc_active = tid < SCROWS && tid >= SCR0;
+  const int sc_cols = sc_row < BM ? p.a_cols : p.b_cols;
+  const int sc_brow = sc_row - BM;                     // weight row of the tile this thread fetches scales for
   const bool sc_second = SWIGLU && sc_brow >= BNC;
-  const __half* const sc_src = (tid < BM ? p.As + (size_t)min(m0 + tid, p.M - 1) * p.a_cols
-                                         : (sc_second ? p.Bs2 : wBs) +
-                                               (size_t)min(n0 + (sc_second ? sc_brow - BNC : sc_brow), wN - 1) * p.b_cols);
-  auto sc_issue = [&](int blk) {
+  const unsigned short* const sc_src =
+      (const unsigned short*)(sc_row < BM ? p.As + (size_t)min(m0 + sc_row, p.M - 1) * p.a_cols
+                                          : (sc_second ? p.Bs2 : wBs) +
+                                                (size_t)min(n0 + (sc_second ? sc_brow - BNC : sc_brow), wN - 1) * p.b_cols);
+  // 16-byte requests need dword-aligned rows of at least eight scales; decided per launch and operand, so that every
+  // thread of the workgroup derives the same first group of a block
+  const int ng = p.K / 128;
+  auto runs_ok = [&](const void* base, int cols) { return cols >= 8 && !(cols & 1) && !((uintptr_t)base & 3); };
+  const bool fast_a = token_scale || runs_ok(p.As, p.a_cols);
+  const bool fast_b = runs_ok(wBs, p.b_cols) && (!SWIGLU || runs_ok(p.Bs2, p.b_cols));
+  auto first_of = [&](int blk, bool fast) { return fast ? min(8 * blk, ng - 8) : 8 * blk; };   // first group of a block
+  v4i sraw = {0, 0, 0, 0};                             // eight scales, two per register
+  auto sc_issue = [&](int blk) __attribute__((always_inline)) {
+    if (sc_active) {
+      const bool fast = sc_row < BM ? fast_a : fast_b;
+      const int g0 = first_of(blk, fast);
+      if (fast) {
+        __builtin_memcpy(&sraw, __builtin_assume_aligned(sc_src + g0, 4), 16);
+      } else {
 #pragma unroll
-    for (int i = 0; i < 8; ++i) sraw[i] = ((const unsigned short*)sc_src)[min(blk * 8 + i, sc_cols - 1)];
-  };
-  auto sc_store = [&](int blk) {
-    if (sc_thread) {
-#pragma unroll
-      for (int i = 0; i < 8; ++i) ((unsigned short*)sc)[((blk & 1) * 8 + i) * SCROWS + tid] = sraw[i];
-    }
-  };
-  // One group: each 32 x 32 tile's two MFMAs start from zero, and the exact sums are folded into the float32
-  // result at once -- out = fma(sum, a_g * b_g, out) (token scale: fma(sum, b_g, out)) in ascending g, which is
-  // the int8 kernel's arithmetic without its int -> float conversion
-  auto mfma_fold = [&](int par, int kt) {
-    const __half* sg = sc + (((kt >> 3) & 1) * 8 + (kt & 7)) * SCROWS;
-    const v16f zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-    auto tile_sum = [&](int i, int j) {
-      v16f t = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(operand(par, TM + j, 0), operand(par, i, 0), zero, kBf6,
-                                                              kBf6, 0, 0, 0, 0);
-      return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(operand(par, TM + j, 1), operand(par, i, 1), t, kBf6, kBf6,
-                                                             0, 0, 0, 0);
-    };
-    // this group's weight scales of the wave tile's columns, converted once for all row blocks
-    float sbf[TN][16];
-#pragma unroll
-    for (int j = 0; j < TN; ++j)
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const h4 b4 = *(const h4*)(sg + BM + wn + j * 32 + 8 * q + 4 * frag_chunk);
-#pragma unroll
-        for (int e = 0; e < 4; ++e) sbf[j][4 * q + e] = (float)b4[e];
+        for (int i = 0; i < 4; ++i)
+          sraw[i] = (int)((unsigned)sc_src[min(g0 + 2 * i, sc_cols - 1)] | (unsigned)sc_src[min(g0 + 2 * i + 1, sc_cols - 1)] << 16);
       }
-    auto fold = [&](int i, int j, const v16f& t) {
-      const float sa = token_scale ? 1.f : __half2float(sg[wm + i * 32 + frag_row]);
-#pragma unroll
-      for (int r = 0; r < 16; ++r)
-        acc[i][j][r] = __builtin_fmaf(t[r], token_scale ? sbf[j][r] : sa * sbf[j][r], acc[i][j][r]);
-    };
-    // the MFMAs of tile n + 1 are issued together with the fold of tile n; a scheduling barrier after each
-    // such pair keeps at most two tiles of sums alive (more would not fit the register file)
-    v16f prev = tile_sum(0, 0);
-#pragma unroll
-    for (int n = 1; n < TM * TN; ++n) {
-      const v16f cur = tile_sum(n / TN, n % TN);
-      fold((n - 1) / TN, (n - 1) % TN, prev);
-      __builtin_amdgcn_sched_barrier(0);
-      prev = cur;
     }
-    fold(TM - 1, TN - 1, prev);
+  };
+  auto sc_store = [&](int blk) __attribute__((always_inline)) {
+    if (sc_active) {
+      unsigned short* dst = (unsigned short*)scl + (blk & 1) * 8 * SCR + (sc_row - SCR0);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) dst[i * SCR] = (unsigned short)((unsigned)sraw[i >> 1] >> (16 * (i & 1)));
+    }
+  };
+  // One group (= one stage): each 32 x 32 tile's two MFMAs start from zero, and the exact sums are folded into the
+  // float32 result -- out = fma(sum, a_g * b_g, out) (token scale: fma(sum, b_g, out)) in ascending g, which is the
+  // int8 kernel's arithmetic without its int -> float conversion.  The fold of a tile is sixteen vector instructions
+  // that must not wait for the tile's own MFMAs, so the tiles form a software pipeline that runs across the stages:
+  // step s issues the two MFMAs of tile s and, between and after them, folds tile s - 1 (whose sums are complete by
+  // then); the last tile of a stage is folded during the first step of the next stage, with the scales of its own
+  // stage kept in registers.  Every accumulator still sees its groups in ascending order.
+  //
+  // Operand roles.  With one scale per row (and for int32 output) the weights are the MFMA's first operand: an output
+  // lane then holds one token (lane % 32) and four consecutive channels per register quad, which packs into 8-byte
+  // writes of the staging tile.  With group scales the activations are the first operand instead: a lane holds one
+  // CHANNEL (lane % 32) and, in register 4 q + e, the token 8 q + 4 (lane / 32) + e of the 32 x 32 tile -- the weight
+  // scale of a group is then one register per lane and column block, and a tile's fold is sixteen plain float32
+  // multiply-adds on it (the mixed-precision multiply-add that would take a half-precision scale straight from a
+  // register issues at half that rate).
+  v16f pend;                                           // sums of the tile whose fold is outstanding: a stage's last
+  float pend_sb = 0.f;                                 // ... the weight scale of the lane's channel in that tile
+  h4 pend_sa[4];                                       // ... and the activation scales of its sixteen tokens (group scales)
+#pragma unroll
+  for (int r = 0; r < 16; ++r) pend[r] = 0.f;
+#pragma unroll
+  for (int q = 0; q < 4; ++q) pend_sa[q] = h4{(_Float16)0.f, (_Float16)0.f, (_Float16)0.f, (_Float16)0.f};
+  auto fold = [&](int i, int j, const v16f& t, float sb, const h4* sa4) __attribute__((always_inline)) {
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        acc[i][j][4 * q + e] = __builtin_fmaf(t[4 * q + e], token_scale ? sb : (float)sa4[q][e] * sb, acc[i][j][4 * q + e]);
+  };
+  constexpr int FOLD_V = token_scale ? 16 : 32;        // vector instructions of one tile's fold
+  // tile n of a stage: row blocks in order, column blocks back and forth; tile 0 is (0, 0)
+  constexpr int LAST = TM * TN - 1;
+  constexpr int LAST_I = LAST / TN, LAST_J = (LAST / TN) & 1 ? TN - 1 - LAST % TN : LAST % TN;
+  auto mfma_fold = [&](auto par_tag, int kt, int stage, int nxt) __attribute__((always_inline)) {
+    constexpr int par = decltype(par_tag)::value;
+    // this step's group inside its block of eight (the last block of a row of scales may start early, see first_of)
+    const int blk = kt >> 3;
+    const __half* sgb = scl + ((blk & 1) * 8 + kt - first_of(blk, fast_b)) * SCR - SCR0;
+    const __half* sga = scl + ((blk & 1) * 8 + kt - first_of(blk, fast_a)) * SCR - SCR0;
+    const v16f zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    // this group's scales, then -- spread over the step -- the next stage's fragments
+    float sb[TN];
+    h4 sa[TM][4];
+#pragma unroll
+    for (int j = 0; j < TN; ++j)   // (kept as a float32 register: folded into the multiply-adds it would make them half rate)
+      sb[j] = round_here(__half2float(sgb[BM + wn + j * 32 + frag_row]));
+    if constexpr (!token_scale) {
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) sa[i][q] = *(const h4*)(sga + wm + i * 32 + 8 * q + 4 * frag_chunk);
+    }
+    read_stage(std::integral_constant<int, par ^ 1>{}, nxt);
+    static_for<TM * TN>([&](auto n_tag) {
+      constexpr int n = decltype(n_tag)::value;
+      constexpr int i = n / TN, j = i & 1 ? TN - 1 - n % TN : n % TN;
+      v16f cur = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(operand(par, i, 0), operand(par, TM + j, 0), zero, kBf6, kBf6,
+                                                                 0, 0, 0, 0);
+      cur = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(operand(par, i, 1), operand(par, TM + j, 1), cur, kBf6, kBf6, 0, 0,
+                                                            0, 0);
+      if constexpr (n == 0) {
+        fold(LAST_I, LAST_J, pend, pend_sb, pend_sa);
+      } else {
+        constexpr int ip = (n - 1) / TN, jp = ip & 1 ? TN - 1 - (n - 1) % TN : (n - 1) % TN;
+        fold(ip, jp, pend, sb[jp], sa[ip]);
+      }
+      pend = cur;
+    });
+    pend_sb = sb[LAST_J];
+    if constexpr (!token_scale) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) pend_sa[q] = sa[LAST_I][q];
+    }
+    // issue order per tile: MFMA, half of the previous tile's fold, MFMA, the other half, with the LDS reads of the next
+    // stage's fragments (four per fragment) spread evenly between them
+    constexpr int NT = TM * TN, RD = 4 * NF, ADDR = 3;
+    static_for<NT>([&](auto n_tag) {
+      constexpr int n = decltype(n_tag)::value;
+      // (ADDR more per slot: the address arithmetic of the fragment reads, which would otherwise pile up behind the
+      // last MFMA)
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x002, FOLD_V / 2 + ADDR, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, RD * (2 * n + 1) / (2 * NT) - RD * (2 * n) / (2 * NT), 0);
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x002, FOLD_V - FOLD_V / 2 + ADDR, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, RD * (2 * n + 2) / (2 * NT) - RD * (2 * n + 1) / (2 * NT), 0);
+    });
   };
 
   // One-scale-per-row epilogue: the tile's scales are fetched now and parked in LDS behind the ring
@@ -264,11 +360,17 @@ void gemm_f6_kernel(const GemmArgs p) {
                             : (e < BM + BN && n < wN ? (second ? p.Bs2 : wBs)[n] : __float2half(1.f));
     }
   }
+  // one scale per token, applied after the groups: the tile's BM of them are parked in LDS behind the group scales now,
+  // so that the epilogue does not start with a round trip to memory per row
+  __half* const tok_sa = scl + 2 * 8 * SCR;            // [BM]
+  if constexpr (token_scale) {
+    if (tid < BM) tok_sa[tid] = p.As[min(m0 + tid, p.M - 1)];
+  }
   if constexpr (GROUPED) sc_issue(0);
 #pragma unroll
   for (int s = 0; s < STAGES - 1; ++s) issue_stage(s, s);
+  if constexpr (GROUPED) sc_store(0);                   // (the compiler waits for its own loads here)
   wait_stages(std::integral_constant<int, STAGES - 2>{});   // stage 0 has landed (this wave's part)
-  if constexpr (GROUPED) sc_store(0);
   if constexpr (EPI == kRowScale) {
 #pragma unroll
     for (int i = 0; i < (BM + BN + T - 1) / T; ++i) {
@@ -277,47 +379,68 @@ void gemm_f6_kernel(const GemmArgs p) {
     }
   }
   __syncthreads();
-  if constexpr (!GROUPED) read_stage(0, 0);
+  read_stage(std::integral_constant<int, 0>{}, 0);
 
-  int stage = 0;
-  // one K step; `par` (a compile-time constant) says which half of the fragment registers feeds the MFMAs
-  auto k_step = [&](auto par_tag, int kt) {
-    constexpr int par = decltype(par_tag)::value;
-    const int nxt = stage + 1 == STAGES ? 0 : stage + 1;
+  // one K step; `par` (a compile-time constant) says which half of the fragment registers feeds the MFMAs, `stage`
+  // which ring slot holds the step's operands, `hook` whether the step also requests (1) or stores (2) the next block
+  // of group scales
+  auto k_step = [&](auto par_tag, auto hook_tag, const int stage, int kt) __attribute__((always_inline)) {
+    constexpr int par = decltype(par_tag)::value, hook = decltype(hook_tag)::value;
+    const int nxt = stage + 1 == STAGES ? 0 : stage + 1, fill = stage == 0 ? STAGES - 1 : stage - 1;
     wait_stages(std::integral_constant<int, STAGES - 3>{});   // this wave's part of stage kt+1 has landed
     // ... everybody's has, and stage kt-1 is free: its fragment reads were consumed an iteration ago; the LDS
     // reads still in flight here belong to stage kt, which nobody overwrites before the next barrier
     barrier_no_fence();
+    // the next block's scales, requested in the previous step (everything outstanding has been waited for); the
+    // buffer they go to was last read in the previous block, which every wave has left by now
+    if constexpr (hook == 2) sc_store((kt >> 3) + 1);
+    issue_stage(fill, kt + STAGES - 1);
+    if constexpr (hook == 1) sc_issue((kt >> 3) + 1);   // ordinary loads; the full wait at the top of the next step covers them
     if constexpr (GROUPED) {
-      // the next block of eight group scales, requested at the end of the previous iteration (everything
-      // outstanding has been waited for above)
-      if ((kt & 7) == 7) sc_store((kt >> 3) + 1);
-    }
-    {
-      int fill = stage + STAGES - 1;
-      if (fill >= STAGES) fill -= STAGES;
-      issue_stage(fill, kt + STAGES - 1);
-    }
-    if constexpr (GROUPED) {
-      // the float32 result doubles the accumulator registers, so the fragments are not double-buffered here: this
-      // stage's are read now, and the other waves of the SIMD cover the LDS latency
-      read_stage(0, stage);
-      mfma_fold(0, kt);
+      mfma_fold(par_tag, kt, stage, nxt);
     } else {
       // fragment reads run one stage ahead of the MFMAs that use them
-      read_stage(par ^ 1, nxt);
+      read_stage(std::integral_constant<int, par ^ 1>{}, nxt);
       mfma_stage(par);
     }
     __builtin_amdgcn_sched_barrier(0);
-    if constexpr (GROUPED) {
-      if (((kt + 1) & 7) == 7) sc_issue(((kt + 1) >> 3) + 1);
-    }
-    stage = nxt;
   };
-  for (int kt = 0; kt < KT; kt += 2) {
-    k_step(std::integral_constant<int, 0>{}, kt);
-    if (kt + 1 < KT) k_step(std::integral_constant<int, 1>{}, kt + 1);
+  constexpr std::integral_constant<int, 0> c0_{};
+  constexpr std::integral_constant<int, 1> c1_{};
+  constexpr std::integral_constant<int, 2> c2_{};
+  int kt = 0;
+  if constexpr (GROUPED) {
+    // blocks of eight steps: the first requests the next block's scales, the second stores them, the others come in
+    // pairs (the fragment parity repeats); the ring slot is a run-time value (with more steps in one block of code the
+    // compiler neither keeps the interleaving nor does without register copies)
+    static_assert(STAGES == 3, "the scale requests rely on the full wait at the top of every step");
+    int stage = 0;
+    auto next = [&]() { stage = stage + 1 == STAGES ? 0 : stage + 1; };
+    while (kt < KT) {
+      const int n = min(8, KT - kt);
+      k_step(c0_, c1_, stage, kt), next();
+      if (n > 1) k_step(c1_, c2_, stage, kt + 1), next();
+      int u = 2;
+      for (; u + 2 <= n; u += 2) {
+        k_step(c0_, c0_, stage, kt + u), next();
+        k_step(c1_, c0_, stage, kt + u + 1), next();
+      }
+      if (u < n) k_step(c0_, c0_, stage, kt + u), next();
+      kt += n;
+    }
+  } else {
+    // as many steps per iteration as it takes for parity and ring slot to repeat: both are compile-time constants then,
+    // every LDS address of a step is a per-lane register that never changes plus an immediate offset, and the loop has no
+    // vector instruction besides the MFMAs
+    constexpr int UNROLL = STAGES % 2 ? 2 * STAGES : STAGES;
+    for (; kt + UNROLL <= KT; kt += UNROLL)
+      static_for<UNROLL>([&](auto u) { k_step(std::integral_constant<int, decltype(u)::value % 2>{}, c0_, decltype(u)::value % STAGES, kt + decltype(u)::value); });
+    static_for<UNROLL - 1>([&](auto u) {               // the remaining steps
+      if (kt + decltype(u)::value < KT)
+        k_step(std::integral_constant<int, decltype(u)::value % 2>{}, c0_, decltype(u)::value % STAGES, kt + decltype(u)::value);
+    });
   }
+  if constexpr (GROUPED) fold(LAST_I, LAST_J, pend, pend_sb, pend_sa);   // the last stage's last tile
   wait_vmcnt<0>();                                    // drain the trailing reloads
   __syncthreads();                                    // every wave is done with the ring
 
@@ -346,37 +469,44 @@ void gemm_f6_kernel(const GemmArgs p) {
   } else {
     // dequantise into this wave's private [WM][WN] fp16 tile in LDS ...
     uint8_t* ep = lds + wave * (WM * EPI_PITCH);
+    if constexpr (GROUPED) {
+      // a lane holds one channel and sixteen tokens per 32 x 32 tile (see "operand roles" above)
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          h4 sa4 = {(_Float16)1.f, (_Float16)1.f, (_Float16)1.f, (_Float16)1.f};
+          if constexpr (token_scale) sa4 = *(const h4*)(tok_sa + wm + i * 32 + 8 * q + 4 * frag_chunk);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const int ml = i * 32 + 8 * q + 4 * frag_chunk + e;   // row inside the wave tile
+#pragma unroll
+            for (int j = 0; j < TN; ++j) {
+              const float f = token_scale ? acc[i][j][4 * q + e] * (float)sa4[e] : acc[i][j][4 * q + e];
+              *(_Float16*)(ep + ml * EPI_PITCH + (j * 32 + frag_row) * 2) = (_Float16)round_here(f);
+            }
+          }
+        }
+    } else {
     float sa[TM];
 #pragma unroll
-    for (int i = 0; i < TM; ++i) {
-      if constexpr (EPI == kRowScale) {
-        sa[i] = __half2float(lds_sa[wm + i * 32 + frag_row]);
-      } else {
-        const int m = m0 + wm + i * 32 + frag_row;
-        sa[i] = token_scale && m < p.M ? __half2float(p.As[m]) : 1.f;
-      }
-    }
+    for (int i = 0; i < TM; ++i) sa[i] = __half2float(lds_sa[wm + i * 32 + frag_row]);
 #pragma unroll
     for (int j = 0; j < TN; ++j)
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
         const int nl = j * 32 + 8 * g + 4 * frag_chunk;   // column inside the wave tile
-        h4 t = {(_Float16)1.0f, (_Float16)1.0f, (_Float16)1.0f, (_Float16)1.0f};
-        if constexpr (EPI == kRowScale) t = *(const h4*)(lds_sa + BM + wn + nl);
+        const h4 t = *(const h4*)(lds_sa + BM + wn + nl);
 #pragma unroll
         for (int i = 0; i < TM; ++i) {
           h4 v;
 #pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            float f;
-            // row scales: float(sum) * (a * b), the scale product is exact, the result rounded once
-            if constexpr (EPI == kRowScale) f = acc[i][j][4 * g + e] * (sa[i] * (float)t[e]);
-            else f = token_scale ? acc[i][j][4 * g + e] * sa[i] : acc[i][j][4 * g + e];
-            v[e] = (_Float16)round_here(f);
-          }
+          for (int e = 0; e < 4; ++e)   // row scales: float(sum) * (a * b), the scale product is exact, the result rounded once
+            v[e] = (_Float16)round_here(acc[i][j][4 * g + e] * (sa[i] * (float)t[e]));
           *(h4*)(ep + (i * 32 + frag_row) * EPI_PITCH + nl * 2) = v;
         }
       }
+    }
     constexpr int CPR = WN / 8, RPI = 64 / CPR;
     const int crow = lane / CPR, cchunk = lane % CPR;
     const bool vec_ok = (wN & 7) == 0;
@@ -512,7 +642,7 @@ int launch_f6(GemmArgs a, hipStream_t stream) {
   }
   a.group_m = a.tiles_m < 4 ? a.tiles_m : 4;
   const size_t smem = (size_t)STAGES * (BM + BN) * kBlockBytes +
-                      (EPI == kRowScale ? (BM + BN) * 2 : (EPI == kGroupScale || EPI == kTokenGroup) ? (BM + BN) * 32 : 0);
+                      (EPI == kRowScale ? (BM + BN) * 2 : EPI == kGroupScale ? (BM + BN) * 32 : EPI == kTokenGroup ? BN * 32 + BM * 2 : 0);
   auto kern = gemm_f6_kernel<BM, BN, WM, WN, STAGES, EPI, SWIGLU, ROPE>;
   static LdsGrant grant;                               // per instantiation
   if (int rc = reserve_lds((const void*)kern, smem, grant, "gemm_f6")) return rc;

@@ -264,8 +264,8 @@ void gemm_i4_kernel(const GemmArgs p) {
                                          : (sc_second ? p.Bs2 : wBs) +
                                                (size_t)min(n0 + (sc_second ? sc_brow - BNC : sc_brow), wN - 1) * p.b_cols);
   // Ordinary loads: the compiler's own wait for them is "everything outstanding", which is what the top
-  // of the next iteration waits for anyway with a three-stage ring -- so they are requested at the end
-  // of one iteration and stored at the top of the next.
+  // of the next iteration waits for anyway with a three-stage ring -- so they are requested in one iteration
+  // (right behind its stage loads) and stored at the top of the next.
   static_assert(!GROUPED || STAGES == 3, "the scale prefetch relies on the full wait at the loop top");
   auto sc_issue = [&](int blk) {
 #pragma unroll
@@ -361,6 +361,11 @@ void gemm_i4_kernel(const GemmArgs p) {
       if (fill >= STAGES) fill -= STAGES;
       issue_stage(fill, kt + STAGES - 1);
     }
+    if constexpr (GROUPED) {
+      // the request for the block of scales after that goes out right behind the stage's loads, one iteration before
+      // its store: it has this whole iteration to arrive, and the full wait at the top of the next one covers it
+      if ((kt + 1) % SPB == SPB - 1) sc_issue((kt + 1) / SPB + 1);
+    }
     if constexpr (GROUPED && GROUP < 128) {
       const uint8_t* st = ring + stage * STAGE;
 #pragma nounroll
@@ -392,9 +397,6 @@ void gemm_i4_kernel(const GemmArgs p) {
       half_step(std::integral_constant<bool, GROUPED>{}, 0, nxt, off_k0);
       half_step(std::false_type{}, 1, nxt, off_k1);
       if constexpr (GROUPED) fold_group(kt, 0);   // one stage is exactly one 128-wide group
-    }
-    if constexpr (GROUPED) {
-      if ((kt + 1) % SPB == SPB - 1) sc_issue((kt + 1) / SPB + 1);
     }
     stage = nxt;
   }

@@ -112,7 +112,8 @@ def test_gemm_f6_argument_errors(ops):
 
 
 @pytest.mark.parametrize("m,n,k", [(1, 128, 128), (33, 200, 640), (300, 384, 2048), (130, 520, 1152), (2048, 1024, 4096),
-                                   (16, 256, 8 * 128), (16, 256, 9 * 128), (700, 4200, 17 * 128)])
+                                   (16, 256, 8 * 128), (16, 256, 9 * 128), (700, 4200, 17 * 128), (64, 256, 18 * 128),
+                                   (130, 260, 11008)])
 @pytest.mark.parametrize("a_token", [False, True])
 def test_gemm_f6_group_scale_equals_the_int8_kernel(ops, m, n, k, a_token):
     """Group scales of 128 on the 6-bit instruction: same bits as the int8 group kernel (both fold
@@ -130,6 +131,10 @@ def test_gemm_f6_group_scale_equals_the_int8_kernel(ops, m, n, k, a_token):
     d6 = ops.gemm_f6_dequant_o16_gs(ops.encode_f6(ap), ops.encode_f6(bp), dev(sa), dev(sb))
     d8 = ops.gemm_i4_dequant(ap, bp, dev(sa), dev(sb), 128)
     assert torch.equal(d6, d8)
+    # the same scales from storage that is only 2-byte aligned (rows of scales are then fetched piece by piece)
+    sa_odd, sb_odd = dev(np.concatenate([[0], sa.ravel()]).astype(np.float16))[1:].view(sa.shape), \
+        dev(np.concatenate([[0], sb.ravel()]).astype(np.float16))[1:].view(sb.shape)
+    assert torch.equal(ops.gemm_f6_dequant_o16_gs(ops.encode_f6(ap), ops.encode_f6(bp), sa_odd, sb_odd), d8)
     if m * n * k <= 300 * 520 * 2048:
         ref, _ = G.gemm_i4_dequant(syn.pack_codes(a), syn.pack_codes(b), sa, sb, group=128)
         assert np.allclose(host(d6).astype(np.float32), ref.astype(np.float32), rtol=1e-3, atol=1e-2)
