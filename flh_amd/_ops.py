@@ -567,11 +567,25 @@ def prefill_attention(q, k_cache, v_cache, past, scale=None):
     return out
 
 
+def _default_attention_workspace(q, need):
+    """The workspace kept per (device, stream) for calls that bring none.  A captured graph keeps the pointer it was
+    recorded with, while this one may be replaced by a larger one later (and a stream handle may be reused by another
+    stream): under capture the caller has to pass a workspace it owns for as long as the graph lives."""
+    _check(not torch.cuda.is_current_stream_capturing(),
+           "decode_attention: pass `workspace` (a tensor that outlives the graph) when capturing")
+    key = (q.device.index, _stream(q))
+    workspace = _attention_workspaces.get(key)
+    if workspace is None or workspace.numel() < need:
+        workspace = torch.empty(max(need, 1 << 20), dtype=torch.uint8, device=q.device)
+        _attention_workspaces[key] = workspace
+    return workspace
+
+
 def decode_attention(q, k_cache, v_cache, kv_len, scale=None, workspace=None):
     """One new token per sequence against the first `kv_len` slots of a preallocated cache: q [B, Hq, d] fp16,
     k_cache / v_cache [B, Hkv, max_len, d] fp16 -> [B, Hq, d] fp16 = softmax(q K^T * scale) V with float32 scores,
     grouped queries (Hq / Hkv in {1, 2, 4, 8}), d in {64, 128}.  `workspace`: a uint8 CUDA tensor for the chunks' partial
-    results; by default one per (device, stream) is kept and grown as needed."""
+    results; by default one per (device, stream) is kept and grown as needed (not under graph capture: pass one then)."""
     for t_ in (q, k_cache, v_cache):
         _check(t_.is_cuda and t_.dtype == torch.float16 and t_.is_contiguous() and t_.device == q.device,
                "tensors must be contiguous float16 CUDA tensors on one device")
@@ -587,13 +601,7 @@ def decode_attention(q, k_cache, v_cache, kv_len, scale=None, workspace=None):
         return out
     need = int(_lib.load().flh_decode_attention_workspace_bytes(B, Hq, d, int(kv_len)))
     if workspace is None:
-        key = (q.device.index, _stream(q))
-        workspace = _attention_workspaces.get(key)
-        if workspace is None or workspace.numel() < need:
-            _check(not torch.cuda.is_current_stream_capturing(),
-                   "decode_attention: call it once eagerly (or pass a workspace) before capturing a graph")
-            workspace = torch.empty(max(need, 1 << 20), dtype=torch.uint8, device=q.device)
-            _attention_workspaces[key] = workspace
+        workspace = _default_attention_workspace(q, need)
     else:
         _check(workspace.is_cuda and workspace.dtype == torch.uint8 and workspace.is_contiguous()
                and workspace.device == q.device and workspace.numel() >= need, f"workspace: {need} bytes of uint8 needed")
@@ -627,13 +635,7 @@ def decode_attention_rope(q, k_new, v_new, cos, sin, positions, k_cache, v_cache
         return out
     need = int(_lib.load().flh_decode_attention_workspace_bytes(B, Hq, d, int(kv_len)))
     if workspace is None:
-        key = (q.device.index, _stream(q))
-        workspace = _attention_workspaces.get(key)
-        if workspace is None or workspace.numel() < need:
-            _check(not torch.cuda.is_current_stream_capturing(),
-                   "decode_attention: call it once eagerly (or pass a workspace) before capturing a graph")
-            workspace = torch.empty(max(need, 1 << 20), dtype=torch.uint8, device=q.device)
-            _attention_workspaces[key] = workspace
+        workspace = _default_attention_workspace(q, need)
     else:
         _check(workspace.is_cuda and workspace.dtype == torch.uint8 and workspace.is_contiguous()
                and workspace.device == q.device and workspace.numel() >= need, f"workspace: {need} bytes of uint8 needed")

@@ -34,7 +34,9 @@ __device__ __forceinline__ _Float16 rope_value(_Float16 x, _Float16 xp, _Float16
 // its position and the cache slot `positions[0]` it takes (the same for every sequence).  The queries are rotated while
 // they are loaded; the workgroup whose chunk holds the slot rotates the new key, uses it and the new value in place of
 // what the cache holds there, and writes both into the cache.  One launch less in front of attention, and the same
-// bytes in the cache as the stand-alone rotary / cache kernel writes.
+// bytes in the cache as the stand-alone rotary / cache kernel writes -- also for a slot in kv_len .. max_len - 1, which
+// attention does not read: the first workgroup of every (sequence, key / value head) writes it there, as the
+// stand-alone kernel would.
 template <int D, int REP, int CHUNK, bool ROPE>
 __global__ __launch_bounds__(kAttnThreads) void decode_attention_partial_kernel(
     const __half* __restrict__ q, __half* k_cache, __half* v_cache, float* __restrict__ partials, uint32_t Hkv,
@@ -57,6 +59,17 @@ __global__ __launch_bounds__(kAttnThreads) void decode_attention_partial_kernel(
   if constexpr (ROPE) {
     const long long pos = positions[0];
     if (pos >= 0 && pos < (long long)kv_len) slot = (uint32_t)pos;
+    if (pos >= (long long)kv_len && pos < (long long)max_len && split == 0 && wave == 0) {
+      // a slot attention does not read: written, not used
+      const _Float16 *kn = (const _Float16*)k_new + (size_t)bh * D, *vn = (const _Float16*)v_new + (size_t)bh * D;
+      const _Float16 *cf = (const _Float16*)cos, *sf = (const _Float16*)sin;
+      _Float16* kd = (_Float16*)k_cache + ((size_t)bh * max_len + (size_t)pos) * D;
+      _Float16* vd = (_Float16*)v_cache + ((size_t)bh * max_len + (size_t)pos) * D;
+      for (int c = lane; c < D; c += 64) {
+        kd[c] = rope_value(kn[c], kn[c ^ (D / 2)], cf[c], sf[c], c < D / 2);
+        vd[c] = vn[c];
+      }
+    }
   }
   const _Float16* qf = (const _Float16*)q + (size_t)bh * REP * D;   // q [B, Hq, D]: the REP heads of this kv head are adjacent
   for (int i = tid; i < REP * D; i += kAttnThreads) {

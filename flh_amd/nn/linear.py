@@ -32,20 +32,26 @@ class LinearFLH(torch.nn.Module):
             self.register_buffer("bias", torch.zeros(out_features, dtype=dtype, device=device))
         else:
             self.bias = None
-        # Opt-in (extension): run prefill-sized calls on the 6-bit matrix instruction.  The weights are then held a
-        # second time, re-encoded at 6 bits per code; outputs are bit-identical.  Pays for wide layers and group scales.
-        # The encoding is rebuilt whenever `w_packed` has been written to or replaced (in-place copies, load_state_dict,
-        # .to(device)): it is keyed on the buffer's storage address and version counter.
-        # The 6-bit matrix instruction for prefill-sized calls (same bits, no unpack in the loop; needs a second, 6-bit
-        # copy of the weights, built on first use): True / False, or None = where it is faster even with the pass that
-        # re-encodes the activations -- weights with a scale per group of 128.
-        self.six_bit = None
+        # Opt-in (extension): run prefill-sized calls on the 6-bit matrix instruction (same bits, no unpack in the loop).
+        # The layer then holds its weights a second time, re-encoded at 6 bits per code: 0.75 byte per weight on top of the
+        # 0.5 of `w_packed`, i.e. 2.5 x the weight memory.  False (default): never.  True: every call of at least
+        # `six_bit_min_rows` rows.  "auto" (or None): where it is faster even with the pass that re-encodes the activations
+        # -- weights with a scale per group of 128.  `prepare_six_bit()` builds the second encoding at once (a loader calls
+        # it); otherwise it is built on first use.  It is rebuilt whenever `w_packed` has been written to or replaced
+        # (in-place copies, load_state_dict, .to(device)): keyed on the buffer's storage address and version counter.
+        self.six_bit = False
         self.six_bit_min_rows = 256
         self._w6 = None
         self._w6_key = None
 
     def drop_six_bit_weights(self):
         self._w6 = self._w6_key = None
+
+    def prepare_six_bit(self):
+        """Build the 6-bit encoding of the weights now if this layer's setting can make use of it (at load time, rather
+        than inside the first long call)."""
+        if self.wants_six_bit(self.six_bit_min_rows):
+            self._six_bit_weights()
 
     def _six_bit_weights(self):
         key = (self.w_packed.data_ptr(), self.w_packed._version, self.w_packed.device)

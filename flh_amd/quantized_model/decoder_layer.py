@@ -74,14 +74,22 @@ def _rotate_half(x):
 
 class StaticKVCache:
     """Preallocated fp16 keys / values [layers][batch, kv_heads, max_len, head_dim].  `layer(i)` is what a decoder layer
-    takes as `kv_cache`: new keys / values are written in place at `positions` (a device index tensor, so a captured
-    graph can be replayed for other positions by overwriting it) and attention reads the first `kv_len` slots."""
+    takes as `kv_cache`: new keys / values are written in place at `positions` and attention reads the first `kv_len`
+    slots, causally for the last T of them.
+
+    The contract between the two: a step over T new tokens runs with ``positions == arange(kv_len - T, kv_len)`` -- the
+    new tokens take the last T of the slots attention reads.  `kv_len` is a host value and the causal structure is
+    derived from it, not from `positions` (a device tensor the host does not read): other positions would let queries
+    see slots that are not theirs to see, or leave the new keys outside what attention reads.  `advance(T)` sets both
+    together.  For the same reason a captured graph serves ONE `kv_len` (it is a launch parameter, fixed at capture):
+    replaying it after overwriting `positions` does not move the range attention reads -- capture one graph per length."""
 
     def __init__(self, layers, batch, kv_heads, max_len, head_dim, device, dtype=torch.float16, q_heads=None):
         self.keys = [torch.zeros(batch, kv_heads, max_len, head_dim, dtype=dtype, device=device) for _ in range(layers)]
         self.values = [torch.zeros_like(k) for k in self.keys]
         self.max_len = max_len
         self.kv_len = 0
+        self._positions = torch.arange(max_len, dtype=torch.int64, device=device)   # advance() hands out views of it
         # the decode-attention kernel's scratch (partial results of the chunks), shared by the layers: they run in
         # order on one stream.  Owned here so that a captured graph finds it allocated.
         q_heads = q_heads or kv_heads * 8
@@ -102,6 +110,14 @@ class StaticKVCache:
 
         def tensors(self):
             return self.owner.keys[self.index], self.owner.values[self.index]
+
+    def advance(self, t):
+        """Make room for `t` new tokens behind what the cache holds: kv_len grows by t; returns the positions
+        arange(kv_len - t, kv_len) (device int64 [t]) the step has to be run with."""
+        if t < 1 or self.kv_len + t > self.max_len:
+            raise ValueError(f"cannot advance a cache of {self.max_len} slots holding {self.kv_len} by {t}")
+        self.kv_len += t
+        return self._positions[self.kv_len - t:self.kv_len]
 
     def layer(self, index):
         return StaticKVCache._Layer(self, index)
@@ -150,11 +166,13 @@ class W4A4DecoderLayer(torch.nn.Module):
 
     @classmethod
     def from_float(cls, weights, num_heads, num_kv_heads, eps=1e-5, act_group_size=128, weight_group_size=None,
-                   fused=True, activation="group", six_bit=None):
+                   fused=True, activation="group", six_bit=False):
         """weights: fp16 tensors `q_proj` ... `down_proj` [N, K] (as nn.Linear stores them) and optionally
         `input_layernorm` / `post_attention_layernorm` [hidden]; quantised round-to-nearest ("group": as they are,
         "token": after the rotation of their input side).  weight_group_size: None = 128 for "group" and one scale
-        per output channel for "token"; 128 with "token" is the Llama-3 arrangement; <= 0 one scale per channel."""
+        per output channel for "token"; 128 with "token" is the Llama-3 arrangement; <= 0 one scale per channel.
+        six_bit: LinearFLH.six_bit of the seven projections -- False (default), True or "auto" (group-scaled weights);
+        anything but False costs a second copy of the weights (2.5 x the weight memory), built here."""
         hidden, inter = weights["q_proj"].size(1), weights["gate_proj"].size(0)
         device = weights["q_proj"].device
         if weight_group_size is None:
@@ -175,9 +193,7 @@ class W4A4DecoderLayer(torch.nn.Module):
             src.weight.data.copy_(w)
             setattr(layer, name, LinearFLH.from_float(src, weight_group_size=weight_group_size,
                                                       in_group_size=act_group_size, no_hadamard=True))
-        if six_bit is not None:   # True: prefill-sized calls on the 6-bit matrix instruction (second encoding of the
-            for name in cls.PROJECTIONS:   # weights); False: never; None: LinearFLH's own choice (group-scaled weights)
-                getattr(layer, name).six_bit = six_bit
+        layer.set_six_bit(six_bit)
         for name in ("input_layernorm", "post_attention_layernorm"):
             norm = getattr(layer, name).to(device)
             if name in weights:
@@ -201,6 +217,15 @@ class W4A4DecoderLayer(torch.nn.Module):
         return hit[1]
 
     _F6_WIDTHS = (512, 1024, 2048, 4096, 8192, 11008, 14336)
+
+    def set_six_bit(self, six_bit):
+        """LinearFLH.six_bit of the seven projections (False, True, or "auto" / None), with the second encoding of the
+        weights built at once where the setting can use it."""
+        for name in self.PROJECTIONS:
+            lin = getattr(self, name)
+            lin.six_bit = None if six_bit == "auto" else six_bit
+            if lin.w_packed.is_cuda:
+                lin.prepare_six_bit()
 
     def _six_bit_for(self, consumers, n_rows, width):
         """Whether the quantiser in front of `consumers` should write the 6-bit operand format directly: every consumer
@@ -275,8 +300,9 @@ class W4A4DecoderLayer(torch.nn.Module):
     def attention(self, x, cos, sin, kv_cache=None, positions=None):
         """x [B, T, hidden] fp16 (already the residual stream); cos / sin [T, head_dim] of the T new positions;
         kv_cache: None, a pair (keys, values) [B, kv_heads, past, head_dim] that grows by concatenation, or one layer
-        of a StaticKVCache together with `positions` (device int64 [T]: the slots the new tokens take; the cache's
-        kv_len says how many slots attention reads).  Causal over past + T positions."""
+        of a StaticKVCache together with `positions` (device int64 [T]: the slots the new tokens take, which must be
+        arange(kv_len - T, kv_len) for the cache's kv_len, the number of slots attention reads -- see StaticKVCache).
+        Causal over past + T positions."""
         _, y, cache = self._attention(x, None, cos, sin, kv_cache, positions, fold_residual=False)
         return y, cache
 

@@ -69,9 +69,9 @@ class W4A4LlamaModel(torch.nn.Module):
         self.lm_head = torch.nn.Linear(shape.hidden_size, shape.vocab_size, bias=False, device=device, dtype=torch.float16)
 
     @classmethod
-    def random_init(cls, shape, activation="token", weight_group_size=128, fused=True, device="cuda", seed=0):
+    def random_init(cls, shape, activation="token", weight_group_size=128, fused=True, device="cuda", seed=0, six_bit=False):
         """Random fp16 weights ~ N(0, 1/K) per linear (norm weights ~ U(0.5, 1.5)), quantised on the device one layer
-        at a time so that no more than one layer's fp16 weights exist at once."""
+        at a time so that no more than one layer's fp16 weights exist at once.  `six_bit`: see set_six_bit."""
         model = cls(shape, activation, weight_group_size, fused, device="meta")
         model.embed_tokens = torch.nn.Embedding(shape.vocab_size, shape.hidden_size, device=device, dtype=torch.float16)
         model.lm_head = torch.nn.Linear(shape.hidden_size, shape.vocab_size, bias=False, device=device, dtype=torch.float16)
@@ -95,7 +95,7 @@ class W4A4LlamaModel(torch.nn.Module):
                     w[name] = (torch.rand(shape.hidden_size, device=device, generator=gen) + 0.5).half()
                 layers.append(W4A4DecoderLayer.from_float(w, shape.num_heads, shape.num_kv_heads, shape.eps, 128,
                                                           weight_group_size if activation == "token" else 128, fused,
-                                                          activation))
+                                                          activation, six_bit))
                 del w
             model.layers = torch.nn.ModuleList(layers)
         return model
@@ -157,10 +157,19 @@ class W4A4LlamaModel(torch.nn.Module):
                        "flh_activation": self.activation}, f, indent=2)
 
     @classmethod
-    def from_quantized(cls, load_directory, device="cuda", activation=None, fused=True):
+    def from_quantized(cls, load_directory, device="cuda", activation=None, fused=True, six_bit=False,
+                       assume_symmetric_weights=False):
         """Build the model a checkpoint directory describes and load its tensors (modeling_llama.py:1139-1260).  The file
         is read without executing anything from it (flh_amd.nn.checkpoint.read_state_dict).  `activation`: "group" (the
-        reference's own models) or "token"; default: what the directory's config says, else "group"."""
+        reference's own models) or "token"; default: what the directory's config says, else "group".  `six_bit`: see
+        set_six_bit.
+
+        Weight symmetry.  This path has kernels for symmetric codes only (signed nibbles, `w_zero` unused).  A directory
+        whose quantization_config.json says `weight_sym: false` -- or lacks the key, which the reference's loader reads as
+        false (modeling_llama.py:1153) -- is refused: the reference's default flow (from_float / save_quantized) writes
+        exactly that flag, although its kernel forward never reads `w_zero` (flh/nn/linear.py:125-132) and the stored
+        nibbles may well be what this path expects.  A caller who knows that the stored codes are signed nibbles with
+        `w_zero` unused passes `assume_symmetric_weights=True`."""
         from ..nn.checkpoint import read_state_dict
         with open(os.path.join(load_directory, "config.json")) as f:
             cfg = json.load(f)
@@ -169,8 +178,12 @@ class W4A4LlamaModel(torch.nn.Module):
         for key, want in (("weight_bits", 4), ("act_bits", 4)):
             if quant.get(key, want) != want:
                 raise ValueError(f"{key} = {quant[key]}: this path is W4A4")
-        if not quant.get("weight_sym", True) or not quant.get("act_sym", True):
-            raise ValueError("asymmetric quantisation has no kernel on this path")
+        if not quant.get("act_sym", True):
+            raise ValueError("asymmetric activation quantisation has no kernel on this path")
+        if not quant.get("weight_sym", False) and not assume_symmetric_weights:
+            raise ValueError("quantization_config.json does not say weight_sym: true (a missing key means false, as in the "
+                             "reference's loader); asymmetric weight codes have no kernel on this path -- pass "
+                             "assume_symmetric_weights=True if the stored codes are signed nibbles with w_zero unused")
         shape = LlamaShape(cfg["hidden_size"], cfg["num_attention_heads"],
                            cfg.get("num_key_value_heads", cfg["num_attention_heads"]), cfg["intermediate_size"],
                            cfg["num_hidden_layers"], cfg["vocab_size"], cfg.get("rms_norm_eps", 1e-5),
@@ -178,15 +191,17 @@ class W4A4LlamaModel(torch.nn.Module):
         activation = activation or cfg.get("flh_activation", "group")
         model = cls(shape, activation, quant.get("weight_group_size", 128), fused, device="cpu")
         model.load_reference_state_dict(read_state_dict(os.path.join(load_directory, "model.pt")))
-        return model.to(device)
+        model = model.to(device)
+        model.set_six_bit(six_bit)
+        return model
 
     @classmethod
-    def from_float(cls, state, shape, activation="token", weight_group_size=128, fused=True, device="cuda"):
+    def from_float(cls, state, shape, activation="token", weight_group_size=128, fused=True, device="cuda", six_bit=False):
         """Quantise a float Llama checkpoint given as a state dict with the transformers key names
         (`model.layers.N.self_attn.q_proj.weight`, ..., `model.embed_tokens.weight`, `model.norm.weight`, `lm_head.weight`):
         round-to-nearest through the same kernels a loader of quantised weights uses, one layer on the device at a time
         (what the reference's `quantize` does layer by layer, modeling_llama.py:789-868, without its GPTQ option -- that is
-        flh_amd.nn.FLHGPTQ on a layer's float weights before this call)."""
+        flh_amd.nn.FLHGPTQ on a layer's float weights before this call).  `six_bit`: see set_six_bit."""
         model = cls(shape, activation, weight_group_size, fused, device="meta")
         emb = state["model.embed_tokens.weight"]
         model.embed_tokens = torch.nn.Embedding(shape.vocab_size, shape.hidden_size, device=device, dtype=torch.float16)
@@ -204,10 +219,18 @@ class W4A4LlamaModel(torch.nn.Module):
                 for name in ("input_layernorm", "post_attention_layernorm"):
                     w[name] = state[pre + name + ".weight"].to(device).half()
                 layers.append(W4A4DecoderLayer.from_float(w, shape.num_heads, shape.num_kv_heads, shape.eps, 128,
-                                                          weight_group_size, fused, activation))
+                                                          weight_group_size, fused, activation, six_bit))
                 del w
         model.layers = torch.nn.ModuleList(layers)
         return model
+
+    def set_six_bit(self, six_bit):
+        """Whether prefill-sized calls of the layers' linears run on the 6-bit matrix instruction: False (default), True,
+        or "auto" (only where it pays even with a re-encoding pass: weights with a scale per group of 128).  Anything but
+        False makes every such linear hold a second, 6-bit copy of its weights -- 0.75 byte per weight on top of 0.5,
+        about + 5 GB for a 7B model -- which is built here, not inside the first long call."""
+        for layer in self.layers:
+            layer.set_six_bit(six_bit)
 
     def new_cache(self, batch, max_len):
         s = self.shape
@@ -235,8 +258,17 @@ class W4A4LlamaModel(torch.nn.Module):
 
     def forward(self, input_ids, positions, cache=None, return_hidden=False):
         """input_ids [B, T] int64, positions [T] int64 (the same for every sequence of the batch).  cache: None (a
-        fresh prefill without cache), or a StaticKVCache whose kv_len the caller has set to the number of slots
-        attention may read (>= positions.max() + 1).  Returns logits [B, T, vocab] fp16 (or the final hidden state)."""
+        fresh prefill without cache), or a StaticKVCache whose kv_len is the number of slots attention reads, with
+        positions == arange(kv_len - T, kv_len) (what cache.advance(T) returns; see StaticKVCache for why nothing else
+        is meaningful).  Returns logits [B, T, vocab] fp16 (or the final hidden state)."""
+        if cache is not None:
+            t = input_ids.size(1)
+            if positions.numel() != t or not 0 < t <= cache.kv_len <= cache.max_len:
+                raise ValueError(f"a step over {t} tokens needs {t} positions and a cache with {t} <= kv_len "
+                                 f"({cache.kv_len}) <= max_len ({cache.max_len})")
+            if not torch.cuda.is_current_stream_capturing() and not torch.equal(
+                    positions, torch.arange(cache.kv_len - t, cache.kv_len, dtype=positions.dtype, device=positions.device)):
+                raise ValueError("positions must be arange(kv_len - T, kv_len) of the cache (cache.advance(T) returns them)")
         x = self.embed(input_ids)
         cos, sin = self._rotary(positions, cache)
         pending = None            # the last MLP output, added inside the next layer's first launch
@@ -262,7 +294,9 @@ class W4A4LlamaModel(torch.nn.Module):
     def capture_decode_step(self, batch, kv_len, cache=None, with_head=True):
         """Record one decode step (batch x 1 token, attention over `kv_len` cached positions, the new token in slot
         kv_len - 1) into a graph.  Returns (graph, static): `static` holds the input ids, the position tensor and the
-        output logits the replays read and write; the cache must already hold the earlier positions."""
+        output logits the replays read and write; the cache must already hold the earlier positions.  The graph serves
+        this kv_len only (the range attention reads is a launch parameter): a replay for another length needs a graph of
+        its own, and `static["positions"]` is to be left at kv_len - 1."""
         dev = self.embed_tokens.weight.device
         cache = cache if cache is not None else self.new_cache(batch, kv_len)
         cache.kv_len = kv_len

@@ -27,7 +27,6 @@ def test_decode_attention_against_float64(b, hq, hkv, d, kv_len, max_len):
     k[:, :, kv_len:] = 100.0                                           # slots past kv_len must not be looked at
     v[:, :, kv_len:] = float("nan")
     print(f"case decode attention b={b} hq={hq} hkv={hkv} d={d} kv_len={kv_len}", flush=True)
-    need = _ops.gemm_i4_workspace_bytes if False else None
     ws = torch.full((int(_ops._lib.load().flh_decode_attention_workspace_bytes(b, hq, d, kv_len)) + 64,), 0xFF,
                     dtype=torch.uint8, device="cuda")                  # NaN patterns: nothing may be read before written
     out = _ops.decode_attention(q, k, v, kv_len, workspace=ws)
@@ -69,11 +68,13 @@ def test_decode_attention_argument_errors():
 @pytest.mark.parametrize("b,hq,hkv,d,kv_len,max_len,slot", [(1, 32, 8, 128, 2048, 2048, 2047), (16, 32, 8, 128, 2048, 2048, 2047),
                                                             (3, 32, 32, 128, 777, 1024, 776), (2, 8, 4, 64, 65, 128, 64),
                                                             (2, 8, 1, 128, 1, 64, 0), (2, 16, 8, 64, 130, 256, 70),
-                                                            (2, 8, 8, 128, 200, 256, 63)])
+                                                            (2, 8, 8, 128, 200, 256, 63), (2, 8, 4, 64, 65, 128, 100),
+                                                            (1, 32, 8, 128, 100, 256, 255)])
 def test_rotary_and_cache_write_inside_attention_give_the_separate_launches_bits(b, hq, hkv, d, kv_len, max_len, slot):
     """flh_decode_attention_rope_f16 against flh_rope_kv_cache_f16 followed by flh_decode_attention_f16 on copies of the
     same cache: the same output, the same cache contents, bit for bit (slot at the end of the live range, at a chunk
-    boundary, in the middle -- an overwrite of an older position -- and slot 0 of an empty cache); q is left alone."""
+    boundary, in the middle -- an overwrite of an older position -- slot 0 of an empty cache, and a slot beyond the
+    live range, which is written and not read); q is left alone."""
     from flh_amd import _ops
     from flh_amd.quantized_model.decoder_layer import rotary_tables
     gen = torch.Generator(device="cuda").manual_seed(kv_len + b + slot)

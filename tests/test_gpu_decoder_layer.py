@@ -123,8 +123,8 @@ def test_six_bit_layer_gives_the_same_bits():
 @pytest.mark.parametrize("six", [None, True])
 def test_token_layer_on_the_six_bit_path_gives_the_same_bits(six):
     """Token configuration with group-scaled weights (the Llama-3 arrangement): from 256 rows on the layer's quantisers
-    write the 6-bit operand format directly and the linears run on the 6-bit matrix instruction (`six_bit=None`: by
-    default for group-scaled weights); outputs and cached keys / values must equal the int8 path's bit for bit."""
+    write the 6-bit operand format directly and the linears run on the 6-bit matrix instruction (`six_bit=None`, the
+    automatic setting: for group-scaled weights); outputs and cached keys / values must equal the int8 path's bit for bit."""
     w, _ = make(seed=21)
     group = 128 if six is None else 0                 # per-channel scales take the 6-bit path only when asked to
     plain = W4A4DecoderLayer.from_float(w, 4, 2, activation="token", weight_group_size=group, six_bit=False)

@@ -353,10 +353,17 @@ def test_float_checkpoint_to_quantised_directory_and_back(tmp_path, activation, 
         # a decode step from a static cache filled by the prefill
         for m, ref in ((model, None), (again, None)):
             cache = m.new_cache(2, 64)
-            cache.kv_len = 40
+            assert torch.equal(cache.advance(40), pos) and cache.kv_len == 40
             m(ids, pos, cache)
-            cache.kv_len = 41
-            step = m(ids[:, :1], torch.tensor([40], device="cuda"), cache)
+            step = m(ids[:, :1], cache.advance(1), cache)
+            assert cache.kv_len == 41
             if m is model:
                 first = step
         assert torch.equal(first, step)
+        # positions that are not the last T slots of what attention reads are refused, as is a cache that cannot grow
+        with pytest.raises(ValueError):
+            model(ids[:, :1], torch.tensor([17], device="cuda"), cache)
+        with pytest.raises(ValueError):
+            model(ids[:, :2], torch.tensor([40], device="cuda"), cache)
+        with pytest.raises(ValueError):
+            cache.advance(64)

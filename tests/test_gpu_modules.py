@@ -250,7 +250,7 @@ def test_six_bit_quantiser_feeds_linear_flh(had):
     assert layer._w6 is None
     got = layer(q6, s6, z6, x_is_packed=True)
     assert got.shape == want.shape and torch.equal(got, want)
-    layer.six_bit = None           # the default: group-scaled weights take the 6-bit instruction from 256 rows on
+    layer.six_bit = None           # automatic: group-scaled weights take the 6-bit instruction from 256 rows on
     assert torch.equal(layer(q4, s4, z4, x_is_packed=True), want)
 
 

@@ -13,7 +13,8 @@ def rot_half(x):
     return torch.cat((-x[..., h:], x[..., :h]), dim=-1)
 
 
-@pytest.mark.parametrize("b,t,hq,hkv,d", [(1, 1, 32, 8, 128), (16, 1, 32, 8, 128), (2, 37, 4, 2, 64), (3, 5, 8, 8, 128)])
+@pytest.mark.parametrize("b,t,hq,hkv,d", [(1, 1, 32, 8, 128), (16, 1, 32, 8, 128), (2, 37, 4, 2, 64), (3, 5, 8, 8, 128),
+                                           (2, 19, 6, 3, 96), (1, 33, 5, 1, 80), (2, 7, 3, 3, 144)])
 @pytest.mark.parametrize("route", ["ext", "ctypes"])
 def test_rope_and_cache_write(b, t, hq, hkv, d, route):
     import flh_amd

@@ -386,8 +386,17 @@ def test_model_checkpoint_directory_uses_the_references_key_names(tmp_path):
     assert again.shape.num_kv_heads == 2 and again.shape.eps == 1e-6 and again.activation == "group"
     a, b = model.state_dict(), again.state_dict()
     assert set(a) == set(b) and all(torch.equal(a[k], b[k]) for k in a)
+    # weight_sym false, or absent (which the reference's loader reads as false): refused unless the caller vouches
+    # that the stored codes are signed nibbles
+    import pytest
+    qc = json.load(open(tmp_path / "quantization_config.json"))
+    for variant in ({**qc, "weight_sym": False}, {k: v for k, v in qc.items() if k != "weight_sym"}):
+        json.dump(variant, open(tmp_path / "quantization_config.json", "w"))
+        with pytest.raises(ValueError, match="weight_sym"):
+            W4A4LlamaModel.from_quantized(tmp_path, device="cpu")
+        vouched = W4A4LlamaModel.from_quantized(tmp_path, device="cpu", assume_symmetric_weights=True).state_dict()
+        assert all(torch.equal(a[k], vouched[k]) for k in a)
     # a checkpoint that lacks a tensor is refused
     del raw["model.layers.0.self_attn.k_proj.w_scale"]
-    import pytest
     with pytest.raises(KeyError):
         W4A4LlamaModel(shape, activation="group", device="cpu").load_reference_state_dict(raw)
