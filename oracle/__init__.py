@@ -33,13 +33,14 @@ than "retyping the formula" fixes each function) is listed per module; the summa
                    kernel's ascending-group fp32 accumulation with fused multiply-add.
 * ``layer``     -- a decoder layer / decode step composed of the pieces above with float64 rotary embedding and
                    attention, pinned by special cases (tests/test_oracle_layer.py).
-* ``gptq``      -- GPTQ in the rotated basis in its elimination form, pinned by closed forms and properties
-                   (tests/test_oracle_gptq.py).
+* ``gptq``      -- GPTQ in the rotated basis in its elimination form, pinned by closed forms and properties and by
+                   the reference's own output on eight seeded cases (tests/golden/gptq_vectors.npz, written from
+                   flh/nn/gptq.py on the CPU by tests/golden/make_gptq_vectors.py; tests/test_oracle_gptq.py).
 
 Parity unpinned (no vector of the reference can exist here, and no closed form decides the open choice):
 ``gemm.gemm_i4_dequant`` with group scales beyond rtol 1e-3 / atol 1e-2 (whether the reference's compiler fuses the
 multiply-add of the fold cannot be observed); ``quant.kernel_had_and_quant`` on random data (CUDA-only arithmetic:
 fp16 butterflies and the ``s <= 1e-6`` rule are restated from the kernel's text, pinned on integer and closed-form rows
-only); ``gptq.gptq`` beyond the properties above (the reference's implementation is CUDA-bound and was read, not run).
+only).
 """
 from . import pack, hadamard, quant, gemm, linear  # noqa: F401
