@@ -367,3 +367,78 @@ def test_float_checkpoint_to_quantised_directory_and_back(tmp_path, activation, 
             model(ids[:, :2], torch.tensor([40], device="cuda"), cache)
         with pytest.raises(ValueError):
             cache.advance(64)
+
+
+def test_llama3_32_layer_decode_graph_against_the_oracle():
+    """The step that the benchmark times for the Llama-3-8B decode configuration -- all 32 layers, norm and head, one
+    captured graph, KV length 2048 -- on one sequence: a replay gives the eager step's logits bit for bit, every layer's
+    input is the previous layer's residual stream plus its MLP output (all 32), and layers 0, 15 and 31 are checked stage
+    by stage against the oracle with the device's own inputs and their own cache contents (a cache slot, position or
+    layer-index mix-up that only shows deep in the stack would fail there)."""
+    from oracle import layer as OL
+    from oracle import prologue
+    shape = LlamaShape.llama3_8b(num_layers=32)
+    batch, kv_len = 1, 2048
+    with torch.no_grad():
+        model = W4A4LlamaModel.random_init(shape, activation="token", weight_group_size=128, fused=True, seed=1)
+    gen = torch.Generator(device="cuda").manual_seed(77)
+    cache = model.new_cache(batch, kv_len)
+    for i in range(shape.num_layers):       # every layer its own contents
+        cache.keys[i][:, :, :kv_len - 1].normal_(0.0, 0.25, generator=gen)
+        cache.values[i][:, :, :kv_len - 1].normal_(0.0, 1.0, generator=gen)
+    tapped = (0, 15, 31)
+    past = {i: (host(cache.keys[i][:, :, :kv_len - 1]), host(cache.values[i][:, :, :kv_len - 1])) for i in tapped}
+    print("case llama3 32-layer decode graph", flush=True)
+    graph, st = model.capture_decode_step(batch, kv_len, cache=cache)
+    ids = torch.randint(0, shape.vocab_size, (batch, 1), device="cuda", generator=gen)
+    st["input_ids"].copy_(ids)
+    torch.cuda.synchronize()
+    graph.replay()
+    torch.cuda.synchronize()
+    replayed = st["output"].clone()
+    graph.replay()                          # a second replay rewrites the same slots with the same values
+    torch.cuda.synchronize()
+    assert torch.equal(st["output"], replayed)
+    recs = [dict() for _ in model.layers]
+    for layer, r in zip(model.layers, recs):
+        layer.record = r
+    with torch.no_grad():
+        hidden_rec = model(ids, st["positions"], cache, return_hidden=True)
+    for layer in model.layers:
+        layer.record = None
+    with torch.no_grad():
+        logits = model(ids, st["positions"], cache)
+        hidden = model(ids, st["positions"], cache, return_hidden=True)
+    assert torch.equal(hidden, hidden_rec), "the single-launch decode path must give the recorded path's bits"
+    assert torch.equal(replayed, logits), "a graph replay must give the eager step's logits"
+    assert torch.isfinite(logits).all()
+    # the residual stream through all 32 layers, from the recorded tensors alone
+    x0 = host(model.embed(ids)).reshape(batch, shape.hidden_size)
+    carried = x0
+    for i, r in enumerate(recs):
+        assert np.array_equal(host(r["attn_in.input"]).reshape(batch, -1), carried), f"input of layer {i}"
+        resid = host(r["mlp_in.input"]).reshape(batch, -1)
+        want = (carried.astype(np.float32) + host(r["o_proj"]).reshape(batch, -1).astype(np.float32)).astype(np.float16)
+        assert np.array_equal(resid, want), f"residual stream behind the attention of layer {i}"
+        carried = (resid.astype(np.float32) + host(r["down_proj"]).reshape(batch, -1).astype(np.float32)).astype(np.float16)
+    fn = host(model.norm.weight).astype(np.float16)
+    want_hidden = prologue.rmsnorm_f16(carried, fn, shape.eps)
+    got_hidden = host(hidden).reshape(batch, -1)
+    assert mismatch(got_hidden.view(np.uint16), want_hidden.view(np.uint16)) < 5e-3
+    sample = np.random.default_rng(3).choice(shape.vocab_size, 2048, replace=False)
+    head = host(model.lm_head.weight[torch.from_numpy(sample).cuda()]).astype(np.float64)
+    assert np.allclose(host(logits).reshape(batch, -1)[:, sample].astype(np.float64), got_hidden.astype(np.float64) @ head.T,
+                       rtol=2e-3, atol=2e-2)
+    # stage by stage, three layers
+    dcos, dsin = rotary_tables(st["positions"], shape.head_dim, shape.rope_theta)
+    cos, sin = host(dcos), host(dsin)
+    for i in tapped:
+        w = oracle_weights(model.layers[i], "token", 128)
+        rec = {k: host(v) for k, v in recs[i].items()}
+        rows = rec["attn_in.input"].reshape(batch, -1)
+        # (this layer's slot kv_len - 1 now holds its new key; the oracle appends its own to the earlier positions)
+        assert np.array_equal(host(cache.keys[i][:, :, :kv_len - 1]), past[i][0])
+        _, report = check_layer_stages(rec, w, rows, cos, sin, batch, 1, past[i], label=f"32-layer graph, layer {i}")
+        print(f"  layer {i}: " + ", ".join(f"{k} {v:.2e}" for k, v in report.items()), flush=True)
+    del model, cache, graph
+    torch.cuda.empty_cache()
