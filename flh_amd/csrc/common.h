@@ -8,6 +8,7 @@
 #include <type_traits>
 
 #include "../../include/flh_hip.h"
+#include "../../include/flh_hip_testing.h"
 
 namespace flh {
 

@@ -132,12 +132,6 @@ int flh_rmsnorm_rotate_quant_gemm_i4_o16_multi(const flh_half* x, const flh_half
                                                const flh_half* const* b_scale, flh_half* const* D, const size_t* N, size_t M,
                                                size_t K, int b_cols, void* stream);
 
-/* Test and tuning hook (no counterpart in the reference): overrides, process-wide, the tile (64, 128 or 256 rows;
- * 0 = automatic) and the split of K inside a workgroup (1, 2 or 4; 0 = automatic) that flh_gemm_i4_o16 and
- * flh_gemm_f6_o16 would choose from the shape.  Every variant gives the same bits; the tests use this to reach
- * all of them.  Combinations a kernel does not offer fall back to the nearest one it does. */
-int flh_gemm_set_tuning(int tile, int k_split);
-
 /* The raw int32 accumulators C[m,n] = sum_k A[m,k] * B[n,k] (for parity checks of the
  * contraction itself; the reference keeps them in registers,
  * flh/kernels/gemm_and_dequant_i4.cu:384-453). */
