@@ -36,11 +36,22 @@ import numpy as np
 
 PEAK_INT8_TOPS = 5033.0   # 256 CU x 8192 int8 op/clk/CU x 2.4 GHz (dense)
 PEAK_HBM_GBS = 8000.0
-# measured HBM traffic per launch at M = 2048 (fetch + write), from the counter runs summarised in
-# profiles/llama7b_block_M2048_hbm_traffic.txt
-GEMM_TRAFFIC_BYTES = {"seven": int(((4 * 40.2 + 2 * 80.2 + 88.2) / 7 + (5 * 16.0 + 2 * 43.0) / 7) * 2 ** 20),
-                      "layer": int(((83.5 + 40.2 + 147.0 + 88.2) / 4 + (48.0 + 16.0 + 43.0 + 16.0) / 4) * 2 ** 20)}
-QUANT4096_TRAFFIC_BYTES = int((16.2 + 4.02) * 2 ** 20)
+# Measured HBM traffic per launch at M = 2048 (fetch + write) is not a constant of this file: it is read from the
+# machine-readable line ("bench.py reads: {...}") of the counter summary committed next to the profiles, so that the
+# figure in the JSON line is the one the committed counter run produced.
+TRAFFIC_FILE = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles", "llama7b_block_M2048_hbm_traffic.txt")
+
+
+def measured_traffic():
+    """{"gemm": {"layer": bytes, "seven": bytes}, "rotate_quant_K4096": bytes} from the counter summary, or None."""
+    try:
+        for line in open(TRAFFIC_FILE):
+            if line.startswith("bench.py reads:"):
+                return json.loads(line.split(":", 1)[1])
+    except (OSError, ValueError):
+        pass
+    return None
+
 
 # (name, N, K, activation source) -- activation sources are quantised once and shared
 LAYERS = [("q", 4096, 4096, "attn_in"), ("k", 4096, 4096, "attn_in"), ("v", 4096, 4096, "attn_in"),
@@ -192,6 +203,8 @@ def main():
                          "(in that order; the run under rocprofv3 --pmc that profiles/ summarises reads its counters per "
                          "dispatch), with the engine clock and socket power rocm-smi reports during each case")
     ap.add_argument("--no-smi", action="store_true", help="with --operand-activity-only: do not start rocm-smi")
+    ap.add_argument("--step-only", type=int, default=0, metavar="STEPS",
+                    help="profiling aid: after the warm-up run exactly STEPS steps of the headline form and exit")
     ap.add_argument("--large-tokens", type=int, default=16384,
                     help="token count of the extra Hadamard-quant launches that amortise the launch floor")
     args = ap.parse_args()
@@ -326,6 +339,21 @@ def main():
             per.setdefault((kind, name), []).append(e0.elapsed_time(e1) * 1e3)  # us
         return ms, {k: float(np.median(v)) for k, v in per.items()}
 
+    if args.step_only:
+        # profiling aid: warm up, then exactly this many steps of the headline form and nothing else, so that the last
+        # 8 (layer form) / 11 (seven) dispatches per step of a kernel trace are the step's launches in order
+        step = make_step(args.launches)
+        warm_gpu()
+        for _ in range(args.warmup):
+            step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.step_only):
+            step()
+        torch.cuda.synchronize()
+        print(json.dumps({"mode": "step-only", "launches": args.launches, "steps": args.step_only,
+                          "us_per_step": round((time.perf_counter() - t0) / args.step_only * 1e6, 1)}))
+        return
     other_form = "seven" if args.launches == "layer" else "layer"
     # the other form first: the first few hundred launches of a process run below the steady rate (clocks and caches
     # settle for longer than a handful of warm-up steps), which would otherwise be charged to whichever form is timed first
@@ -647,6 +675,46 @@ def main():
         f6[f"{n}x{k}"] = {"us": round(us, 2), "TOPS": round(gemm_ops(M, n, k) / (us * 1e-6) / 1e12, 1),
                           "encode_activations_us": round(us_enc, 2), "equal_to_int8_path": same}
         del w6, a6
+    # The headline step itself on the 6-bit matrix instruction (side figure, never `value`): the quantisers write the
+    # 6-bit operand format directly (matrix-core rotation), weights re-encoded once, the same four launches as the layer
+    # form -- q/k/v in one, o, gate and up in one that stores silu(gate) * up, down.  Same outputs bit for bit.
+    w6_all = {name: ops.encode_f6(weights[name][0]) for name in weights}
+
+    def step_6bit(events=None):
+        out = None
+        for src, parts in (("attn_in", ["q", "k", "v"]), ("attn_out", ["o"]), ("mlp_in", ["gate", "up"]), ("mlp_mid", ["down"])):
+            a6, ps = ops.rotate_and_quantize_f6(acts[src], hadamard=(True if SOURCES[src] != 4096 else "fast"))
+            if events is not None:
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+            if parts == ["gate", "up"]:
+                out = ops.gemm_f6_swiglu(a6, w6_all["gate"], w6_all["up"], ps, weights["gate"][1], weights["up"][1])
+            elif len(parts) == 1:
+                out = ops.gemm_f6_dequant_o16(a6, w6_all[parts[0]], ps, weights[parts[0]][1])
+            else:
+                out = ops.gemm_f6_dequant_multi(a6, [w6_all[n] for n in parts], ps, [weights[n][1] for n in parts])
+            if events is not None:
+                e1.record()
+                events.append((src, e0, e1))
+        return out
+
+    us_step6 = wall_us(step_6bit, reps=args.steps)
+    ev6 = []
+    for _ in range(args.steps):
+        step_6bit(ev6)
+    torch.cuda.synchronize()
+    per6 = {}
+    for src, e0, e1 in ev6:
+        per6.setdefault(src, []).append(e0.elapsed_time(e1) * 1e3)
+    gemm6_us = sum(float(np.median(v)) for v in per6.values())
+    f6["step_in_layer_form"] = {
+        "us_per_layer": round(us_step6, 1),
+        "TOPS": round(sum(gemm_ops(M, n, k) for _, n, k, _ in LAYERS) / (us_step6 * 1e-6) / 1e12, 1),
+        "gemm_launch_us": {src: round(float(np.median(v)), 2) for src, v in per6.items()},
+        "gemm_TOP/s": round(sum(gemm_ops(M, n, k) for _, n, k, _ in LAYERS) / (gemm6_us * 1e-6) / 1e12, 1),
+        "gemm_frac_of_int8_peak": round(sum(gemm_ops(M, n, k) for _, n, k, _ in LAYERS) / (gemm6_us * 1e-6) / 1e12 / PEAK_INT8_TOPS, 4),
+        "note": "v_mfma_f32_32x32x64_f8f6f4 on int4 codes encoded as e3m2 (exact); the headline stays on the int8 instruction"}
+    del w6_all
     # group scales of 128 on the weights, one scale per token (the Llama-3 weight-group configuration), both kernels
     for n, k in ((4096, 4096), (14336, 4096)):
         wq = torch.randint(0, 256, (n, k // 2), dtype=torch.uint8, device=dev)
@@ -711,12 +779,12 @@ def main():
     us = wall_us(llama3_step_6bit, reps=args.steps)
     llama3["six_bit_matrix_instruction"] = {"us_per_layer": round(us, 1), "TOPS": round(ops3 / (us * 1e-6) / 1e12, 1)}
 
-    # ... with the quantisers writing the 6-bit format themselves (no encoding pass; float32 butterflies for K = 4096,
+    # ... with the quantisers writing the 6-bit format themselves (no encoding pass; K = 4096 in the run's rotation mode,
     # matrix cores for K = 14336) and the projections that share an input in one launch: what a token-configuration layer
     # with group-scaled weights issues for 256 rows or more
     def llama3_step_6bit_direct():
         for src, parts in groups3:
-            a6, ps = ops.rotate_and_quantize_f6(acts3[src])
+            a6, ps = ops.rotate_and_quantize_f6(acts3[src], hadamard=(True if L3_SRC[src] != 4096 else had_mode(4096)))
             out = ops.gemm_f6_dequant_multi(a6, [w3_6[n] for n in parts], ps, [w3[n][1] for n in parts])
         return out
 
@@ -917,20 +985,12 @@ def main():
     # int32 output, no nibble unpacking and no dequantisation) and fp16 GEMM on the same shapes, as a measure
     # of what fraction of the nominal matrix-core peak a tuned GEMM sustains on this device at these sizes
     # Diagnostic, not product: the q / k / v-sized launch on operands of less switching activity.  The part is at its power
-    # limit under this kernel, and how fast it runs depends on how many operand bits toggle: all-zero codes show what the
-    # kernel's structure alone allows, a zero in every other code lies in between; codes quantised from normal data run
-    # within 2 % of uniform random ones.
-    activity = {}
+    # limit under this kernel (rocm-smi reads the cap, 1400 W, and a lowered engine clock), and how fast it runs depends on
+    # how many operand bits toggle: all-zero codes run at the full 2400 MHz and show what the kernel's structure alone
+    # allows, a zero in every other code lies in between; codes quantised from normal data run within 2 % of uniform
+    # random ones.  The launch takes the same number of engine cycles in all three cases (counter run in profiles/).
     n_act, k_act = 12288, 4096
-    sa_act = torch.full((M, 1), 0.01, dtype=torch.float16, device=dev)
-    sb_act = torch.full((n_act, 1), 0.01, dtype=torch.float16, device=dev)
-    for label, hi in (("uniform_random_codes", 256), ("every_other_code_zero", 16), ("all_zero_codes", 1)):
-        a_act = torch.randint(0, hi, (M, k_act // 2), dtype=torch.uint8, device=dev)
-        b_act = torch.randint(0, hi, (n_act, k_act // 2), dtype=torch.uint8, device=dev)
-        us = timed([lambda: ops.gemm_i4_dequant_o16(a_act, b_act, sa_act, sb_act)] * 20)
-        activity[label] = {"us": round(us, 2), "TOPS": round(gemm_ops(M, n_act, k_act) / (us * 1e-6) / 1e12, 1),
-                           "frac_of_peak": round(gemm_ops(M, n_act, k_act) / (us * 1e-6) / 1e12 / PEAK_INT8_TOPS, 4)}
-        del a_act, b_act
+    activity = operand_activity(torch, ops, M, 20, True)["cases"]   # time, engine clock and socket power per case
     vendor = None
     if not args.no_vendor_reference:
         vendor = {}
@@ -960,6 +1020,8 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
+    traffic = measured_traffic()
+    copy_cold = cold[f"K=4096,M={M}"]["device_copy"]
     total_ops = sum(gemm_ops(M, n, k) for _, n, k, _ in LAYERS)
     launches = FORMS[args.launches]
     gemm_us = sum(med[("gemm", name)] for name, *_ in launches)
@@ -990,7 +1052,16 @@ def main():
         "data": "synthetic",
         "config": {"workload": "Llama-2-7B decoder-block linears, M=2048, per-token x per-channel scales "
                                "(the configuration the headline metric is quoted on)", "tokens": M,
-                   "launches": args.launches},
+                   "launches": args.launches, "hadamard": args.hadamard,
+                   "notes": ("the step is issued as a decoder layer issues it: " +
+                             ("FOUR GEMM launches for the seven contractions (q/k/v as three weight matrices of one launch; "
+                              "gate and up as one launch that stores silu(gate)*up instead of the two fp16 outputs), "
+                              if args.launches == "layer" else "one GEMM launch per linear, ") +
+                             f"rotation mode '{args.hadamard}' ('fast' = matrix cores; its code mismatch rates against the "
+                             "exactly rounded transform are reported in roofline_hadamard_quant), and every timed region "
+                             "starts at steady clocks (sustained GEMMs until a batch stops getting faster, then --warmup "
+                             "steps).  The form comparable with one-launch-per-linear figures is 'launches=seven', "
+                             "reported beside this one.")},
         "roofline": {"bound": "mfma",
                      "kernel": "gemm_i4_kernel (row-scale epilogue), " +
                                ("4 launches per step: q/k/v in one, o, gate and up in one (stores silu(gate)*up), down"
@@ -999,7 +1070,7 @@ def main():
                      "frac": round(gemm_tops / PEAK_INT8_TOPS, 4),
                      # HBM bytes per launch averaged over the seven launches (rocprofv3 --pmc FETCH_SIZE and
                      # WRITE_SIZE runs of this script, calibrated on a 256 MiB copy; summary under profiles/)
-                     "traffic": GEMM_TRAFFIC_BYTES[args.launches] if M == 2048 else None,
+                     "traffic": traffic["gemm"][args.launches] if (traffic and M == 2048) else None,
                      "avg_launch_us": round(gemm_us / len(launches), 2),
                      "per_launch": launch_table(args.launches, med),
                      # what the part clocks at under this load, and the fraction of the peak at that clock
@@ -1016,7 +1087,19 @@ def main():
                                                "rotate_quant_wave_kernel<8>") + f" (K=4096, M={M}, inside the step)",
                                     "achieved": round(q4096_gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
                                     "frac": round(q4096_gbs / PEAK_HBM_GBS, 4),
-                                    "traffic": QUANT4096_TRAFFIC_BYTES if M == 2048 else None,
+                                    # what a plain device copy of the same rows reaches on this box in this run (cold
+                                    # inputs, graph replays: no host gaps): the practical ceiling of a streaming launch
+                                    # of this size, and the same kernel's own cold figure against it
+                                    "practical_peak_GB/s": copy_cold["GB/s"],
+                                    "frac_of_practical_peak": round(q4096_gbs / copy_cold["GB/s"], 4),
+                                    "cold_launch_frac_of_practical_peak": round(
+                                        cold[f"K=4096,M={M}"]["fast" if had_mode(4096) == "fast" else "exact"]["GB/s"] / copy_cold["GB/s"], 4),
+                                    f"K=4096,M={ML},cold_frac_of_practical_peak": round(
+                                        cold[f"K=4096,M={ML}"]["fast" if had_mode(4096) == "fast" else "exact"]["GB/s"] /
+                                        cold[f"K=4096,M={ML}"]["device_copy"]["GB/s"], 4),
+                                    "note": "per-launch HIP events around a 7 us kernel also time about 2 us of dispatch: the "
+                                            "profiler's duration of these same launches is 7.2-7.5 us (profiles/)",
+                                    "traffic": traffic["rotate_quant_K4096"] if (traffic and M == 2048) else None,
                                     "avg_launch_us": round(q4096_us, 2), "per_launch": quant_detail,
                                     "hadamard_mode": args.hadamard, "modes_alone": modes,
                                     f"K=4096,M={ML}": large, "cold_inputs_K=4096": cold,
