@@ -32,7 +32,8 @@ def test_static_scratch_entry_point_equals_the_workspace_one():
     lib = _lib.load()
     assert lib.flh_init() == 0, lib.flh_last_error()
     gen = torch.Generator(device="cuda").manual_seed(1)
-    for b, hq, hkv, d, kv_len, max_len in ((16, 32, 8, 128, 2048, 2048), (3, 8, 4, 64, 100, 128)):   # the second smaller
+    for b, hq, hkv, d, kv_len, max_len in ((16, 32, 8, 128, 2048, 2048), (3, 8, 4, 64, 100, 128),   # the second smaller
+                                           (24, 32, 32, 128, 1000, 1024)):                       # ... and a larger one again
         q = torch.randn(b, hq, d, device="cuda", generator=gen).half()
         k = (torch.randn(b, hkv, max_len, d, device="cuda", generator=gen) * 0.5).half()
         v = torch.randn(b, hkv, max_len, d, device="cuda", generator=gen).half()
