@@ -205,6 +205,10 @@ def main():
     ap.add_argument("--no-smi", action="store_true", help="with --operand-activity-only: do not start rocm-smi")
     ap.add_argument("--step-only", type=int, default=0, metavar="STEPS",
                     help="profiling aid: after the warm-up run exactly STEPS steps of the headline form and exit")
+    ap.add_argument("--decode-step-only", type=int, default=0, metavar="REPLAYS",
+                    help="profiling aid: only the 32-layer Llama-3-8B decode step (kv_len 2048) of --decode-batch sequences, "
+                         "captured into a graph and replayed REPLAYS times after five warm replays")
+    ap.add_argument("--decode-batch", type=int, default=1)
     ap.add_argument("--large-tokens", type=int, default=16384,
                     help="token count of the extra Hadamard-quant launches that amortise the launch floor")
     args = ap.parse_args()
@@ -221,6 +225,25 @@ def main():
     M = args.tokens
     if args.operand_activity_only:
         print(json.dumps(operand_activity(torch, ops, M, args.operand_activity_only, not args.no_smi)))
+        return
+    if args.decode_step_only:
+        from flh_amd.quantized_model import LlamaShape, W4A4LlamaModel
+        with torch.no_grad():
+            model = W4A4LlamaModel.random_init(LlamaShape.llama3_8b(num_layers=32), activation="token", weight_group_size=128,
+                                               fused=True, seed=1)
+        graph, state = model.capture_decode_step(args.decode_batch, 2048)
+        for i in range(32):
+            state["cache"].keys[i].normal_()
+            state["cache"].values[i].normal_()
+        for _ in range(5):
+            graph.replay()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.decode_step_only):
+            graph.replay()
+        torch.cuda.synchronize()
+        print(json.dumps({"mode": "decode-step-only", "batch": args.decode_batch, "replays": args.decode_step_only,
+                          "ms_per_step": round((time.perf_counter() - t0) / args.decode_step_only * 1e3, 3)}))
         return
     acts_h, weights_h = make_inputs(M)
     dev = torch.device("cuda:0")
