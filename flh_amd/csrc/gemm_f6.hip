@@ -674,7 +674,13 @@ int launch_f6_swiglu(const GemmArgs& a, hipStream_t stream) {
   auto tiles = [&](int bm, int bnc) { return (long)((a.M + bm - 1) / bm) * ((a.N + bnc - 1) / bnc); };
   int tile = tiles(128, 64) >= 200 ? 128 : 64;
   const int forced = g_tune_tile.load(std::memory_order_relaxed);
+  if constexpr (EPI == kRowScale) {                   // the eight-wave tile: see launch_f6_by_shape
+    if (tiles(256, 64) >= 256) tile = 256;
+    if (forced == 256) tile = 256;
+  }
   if (forced == 128 || forced == 64) tile = forced;
+  if constexpr (EPI == kRowScale)
+    if (tile == 256) return launch_f6<256, 128, 64, 64, 4, EPI, true>(a, stream);
   if (tile == 128) return launch_f6<128, 128, 64, 64, 3, EPI, true>(a, stream);
   return launch_f6<64, 64, 32, 32, 3, EPI, true>(a, stream);
 }
@@ -685,9 +691,13 @@ int launch_f6_by_shape(const GemmArgs& a, hipStream_t stream) {
   const int env_tile = g_tune_tile.load(std::memory_order_relaxed);
   const int n_all = total_n_f6(a);
   auto tiles = [&](int bm, int bn) { return (long)((a.M + bm - 1) / bm) * ((n_all + bn - 1) / bn); };
-  // measured at M = 2048 on the Llama shapes: two 128 x 128 workgroups per compute unit beat one 256 x 128
-  // workgroup of eight waves by 2-10 %; the large tile is kept for the override
-  int tile = tiles(128, 128) >= 256 ? 128 : 64;
+  // Measured at M = 2048 / 4096 on the Llama shapes.  With the same weights launched back to back (they then sit in the
+  // last-level cache) two 128 x 128 workgroups per compute unit beat one 256 x 128 workgroup of eight waves by 2-6 %;
+  // with weights that come from HBM -- every launch of a model, whose layers' weights do not fit that cache -- the
+  // eight-wave tile with its four-stage ring is 12-16 % faster at every shape (gate + up 148 against 170 us, q + k + v
+  // 79 against 90, down 61 against 72, o 27.5 against 31.5): it requests half the operand bytes per unit of matrix
+  // work and a step further ahead.  It is taken as soon as there is one such tile per compute unit.
+  int tile = tiles(256, 128) >= 256 ? 256 : tiles(128, 128) >= 256 ? 128 : 64;
   if (env_tile == 256 || env_tile == 128 || env_tile == 64) tile = env_tile;
   if (tile == 256) return launch_f6<256, 128, 64, 64, 4, EPI>(a, stream);
   if (tile == 128) return launch_f6<128, 128, 64, 64, 3, EPI>(a, stream);
@@ -848,7 +858,13 @@ extern "C" int flh_gemm_f6_qkv_rope_o16(const uint8_t* A6, const flh_half* a_sca
   g.rope_max_len = (int)max_len;
   g.rope_hkv = (int)Hkv;
   // 128 x 128 tiles (a tile column = one head)
-  if (rows_only) return launch_f6<128, 128, 64, 64, 3, kRowScale, false, true>(g, (hipStream_t)stream);
+  if (rows_only) {
+    const int forced = g_tune_tile.load(std::memory_order_relaxed);
+    const long tiles256 = (long)((g.M + 255) / 256) * ((total_n_f6(g) + 127) / 128);
+    if (forced == 256 || (forced == 0 && tiles256 >= 256))
+      return launch_f6<256, 128, 64, 64, 4, kRowScale, false, true>(g, (hipStream_t)stream);
+    return launch_f6<128, 128, 64, 64, 3, kRowScale, false, true>(g, (hipStream_t)stream);
+  }
   if (a_cols == 1) return launch_f6<128, 128, 64, 64, 3, kTokenGroup, false, true>(g, (hipStream_t)stream);
   return launch_f6<128, 128, 64, 64, 3, kGroupScale, false, true>(g, (hipStream_t)stream);
 }

@@ -113,7 +113,8 @@ def test_qkv_rope_gemm_equals_the_two_launches_at_llama_width(ops):
 
 @pytest.mark.parametrize("batch,t,hq,hkv,k", [(1, 70, 4, 4, 256), (3, 50, 4, 2, 512), (2, 300, 8, 2, 384), (1, 5, 2, 1, 128)])
 @pytest.mark.parametrize("scales", ["row", "token_group", "group_group"])
-def test_qkv_rope_gemm_on_the_six_bit_instruction(ops, batch, t, hq, hkv, k, scales):
+@pytest.mark.parametrize("tile", [0, 256])                         # 256: the eight-wave tile of the row-scale launch
+def test_qkv_rope_gemm_on_the_six_bit_instruction(ops, batch, t, hq, hkv, k, scales, tile, gemm_tuning):
     """flh_gemm_f6_qkv_rope_o16: the same queries and cache bytes as the int8 launch (itself checked against the oracle)."""
     from flh_amd.quantized_model import rotary_tables
     a_cols, b_cols = {"row": (1, 1), "token_group": (1, 2), "group_group": (2, 2)}[scales]
@@ -127,7 +128,9 @@ def test_qkv_rope_gemm_on_the_six_bit_instruction(ops, batch, t, hq, hkv, k, sca
     vc = torch.full_like(kc, -3.0)
     kc6, vc6 = kc.clone(), vc.clone()
     q = ops.gemm_i4_qkv_rope(A, S, W, WS, cos, sin, pos, kc, vc, batch)
+    gemm_tuning(tile)
     q6 = ops.gemm_f6_qkv_rope(ops.encode_f6(A), S, [ops.encode_f6(w) for w in W], WS, cos, sin, pos, kc6, vc6, batch)
+    gemm_tuning(0)
     assert torch.equal(q, q6) and torch.equal(kc, kc6) and torch.equal(vc, vc6)
 
 

@@ -123,11 +123,11 @@ def test_swiglu_layer_method_and_errors(ops):
 
 @pytest.mark.parametrize("m,n,k", [(300, 200, 512), (64, 64, 128), (513, 1000, 1024), (2048, 1408, 4096), (130, 36, 384)])
 @pytest.mark.parametrize("a_cols,b_cols", [(1, 1), (1, 2), (2, 2)])
-@pytest.mark.parametrize("tile", [0, 64, 128])
+@pytest.mark.parametrize("tile", [0, 64, 128, 256])            # 256: the eight-wave tile (one scale per row only)
 def test_six_bit_swiglu_gemm_gives_the_int8_launch_bits(ops, gemm_tuning, m, n, k, a_cols, b_cols, tile):
     """flh_gemm_f6_swiglu_o16 on re-encoded operands against flh_gemm_i4_swiglu_o16 on the nibbles: the sums are the same
     integers, the epilogue the same arithmetic, the product the same device routine -- so bit for bit, for every scale
-    layout, ragged M and N, both tiles."""
+    layout, ragged M and N, every tile."""
     print(f"case f6 swiglu m={m} n={n} k={k} a_cols={a_cols} b_cols={b_cols} tile={tile}", flush=True)
     ap, bg, bu, sa, sg, su = case(m, n, k, 31 + m + n, a_cols, b_cols)
     a, g, u = dev(ap), dev(bg), dev(bu)
