@@ -903,6 +903,10 @@ def main():
                 layer.fast_rotation = True
                 layer_fig["token_configuration,prefill_8x512,fused,matrix_core_rotation_us"] = round(
                     wall_us(lambda: layer(xs8, cos8, sin8), reps=20), 1)
+                # ... and with the seven linears on the 6-bit matrix instruction as well (a second encoding of the weights)
+                layer.set_six_bit(True)
+                layer_fig["token_configuration,prefill_8x512,fused,matrix_core_rotation,6bit_matrix_instruction_us"] = round(
+                    wall_us(lambda: layer(xs8, cos8, sin8), reps=20), 1)
             del layer
     del lw, xs, xs8
     # the causal attention kernel of the prefill path alone, beside torch's fused attention on the same tensors
@@ -1084,7 +1088,9 @@ def main():
                              "exactly rounded transform are reported in roofline_hadamard_quant), and every timed region "
                              "starts at steady clocks (sustained GEMMs until a batch stops getting faster, then --warmup "
                              "steps).  The form comparable with one-launch-per-linear figures is 'launches=seven', "
-                             "reported beside this one.")},
+                             "reported beside this one.  The headline runs on the int8 matrix instruction; the same step "
+                             "on the 6-bit one (bit-identical outputs, a second encoding of the weights) is "
+                             "gemm_on_6bit_matrix_instruction.step_in_layer_form.")},
         "roofline": {"bound": "mfma",
                      "kernel": "gemm_i4_kernel (row-scale epilogue), " +
                                ("4 launches per step: q/k/v in one, o, gate and up in one (stores silu(gate)*up), down"
