@@ -695,8 +695,8 @@ int launch_f6_by_shape(const GemmArgs& a, hipStream_t stream) {
   // last-level cache) two 128 x 128 workgroups per compute unit beat one 256 x 128 workgroup of eight waves by 2-6 %;
   // with weights that come from HBM -- every launch of a model, whose layers' weights do not fit that cache -- the
   // eight-wave tile with its four-stage ring is 12-16 % faster at every shape (gate + up 148 against 170 us, q + k + v
-  // 79 against 90, down 61 against 72, o 27.5 against 31.5): it requests half the operand bytes per unit of matrix
-  // work and a step further ahead.  It is taken as soon as there is one such tile per compute unit.
+  // 79 against 90, down 61 against 72, o 27.5 against 31.5): it requests three quarters of the operand bytes per unit
+  // of matrix work and a step further ahead.  It is taken as soon as there is one such tile per compute unit.
   int tile = tiles(256, 128) >= 256 ? 256 : tiles(128, 128) >= 256 ? 128 : 64;
   if (env_tile == 256 || env_tile == 128 || env_tile == 64) tile = env_tile;
   if (tile == 256) return launch_f6<256, 128, 64, 64, 4, EPI>(a, stream);
