@@ -91,6 +91,9 @@ __device__ __forceinline__ void load_to_lds16(const void* sbase, unsigned voffse
 // moving memory operations across it.
 __device__ __forceinline__ void barrier_no_fence() { asm volatile("s_barrier" ::: "memory"); }
 
+// every LDS (and scalar memory) operation of this wave has completed
+__device__ __forceinline__ void wait_lgkmcnt0() { __builtin_amdgcn_s_waitcnt(0xC07F); }
+
 template <int N>
 __device__ __forceinline__ void wait_vmcnt() {
   static_assert(N >= 0 && N < 64, "vmcnt range");

@@ -367,10 +367,19 @@ void gemm_f6_kernel(const GemmArgs p) {
     if (tid < BM) tok_sa[tid] = p.As[min(m0 + tid, p.M - 1)];
   }
   if constexpr (GROUPED) sc_issue(0);
+  // REFILL_OWN (three-stage rings): a stage's fragments are read into registers one step before they are multiplied, so
+  // its slot is free a step before the classic ring order would refill it.  The whole ring is requested up front and a
+  // step refills the slot of the stage it multiplies: every stage then has two steps to arrive instead of one, at the
+  // same LDS footprint -- what weights that come from HBM rather than from the last-level cache need.
+#ifndef FLH_F6_REFILL_OWN
+#define FLH_F6_REFILL_OWN 1
+#endif
+  constexpr bool REFILL_OWN = FLH_F6_REFILL_OWN && STAGES == 3;
+  constexpr int AHEAD = REFILL_OWN ? STAGES : STAGES - 1;   // stages in flight or waiting beyond the one being multiplied
 #pragma unroll
-  for (int s = 0; s < STAGES - 1; ++s) issue_stage(s, s);
+  for (int s = 0; s < AHEAD; ++s) issue_stage(s, s);
   if constexpr (GROUPED) sc_store(0);                   // (the compiler waits for its own loads here)
-  wait_stages(std::integral_constant<int, STAGES - 2>{});   // stage 0 has landed (this wave's part)
+  wait_stages(std::integral_constant<int, AHEAD - 1>{});   // stage 0 has landed (this wave's part)
   if constexpr (EPI == kRowScale) {
 #pragma unroll
     for (int i = 0; i < (BM + BN + T - 1) / T; ++i) {
@@ -387,14 +396,16 @@ void gemm_f6_kernel(const GemmArgs p) {
   auto k_step = [&](auto par_tag, auto hook_tag, const int stage, int kt) __attribute__((always_inline)) {
     constexpr int par = decltype(par_tag)::value, hook = decltype(hook_tag)::value;
     const int nxt = stage + 1 == STAGES ? 0 : stage + 1, fill = stage == 0 ? STAGES - 1 : stage - 1;
-    wait_stages(std::integral_constant<int, STAGES - 3>{});   // this wave's part of stage kt+1 has landed
+    wait_stages(std::integral_constant<int, AHEAD - 2>{});   // this wave's part of stage kt+1 has landed
     // ... everybody's has, and stage kt-1 is free: its fragment reads were consumed an iteration ago; the LDS
-    // reads still in flight here belong to stage kt, which nobody overwrites before the next barrier
+    // reads still in flight here belong to stage kt, which nobody overwrites before the next barrier -- unless this
+    // step refills that very slot: then every wave lets its reads of stage kt finish before it signals
+    if constexpr (REFILL_OWN) wait_lgkmcnt0();
     barrier_no_fence();
     // the next block's scales, requested in the previous step (everything outstanding has been waited for); the
     // buffer they go to was last read in the previous block, which every wave has left by now
     if constexpr (hook == 2) sc_store((kt >> 3) + 1);
-    issue_stage(fill, kt + STAGES - 1);
+    issue_stage(REFILL_OWN ? stage : fill, kt + AHEAD);
     if constexpr (hook == 1) sc_issue((kt >> 3) + 1);   // ordinary loads; the full wait at the top of the next step covers them
     if constexpr (GROUPED) {
       mfma_fold(par_tag, kt, stage, nxt);
