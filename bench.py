@@ -1039,6 +1039,65 @@ def main():
                 "fp16_us": round(us16, 2), "fp16_TFLOPS": round(gemm_ops(M, n, k) / (us16 * 1e-6) / 1e12, 1)}
             del a8, b8, a16, b16
 
+    # The step's four GEMM launches on weights that come from HBM: every launch takes the next of several sets of random
+    # weights, more bytes in all than the 256 MB last-level cache holds (the state a model's layers are in), beside the
+    # same launch on one set launched back to back (cached).  int8 kernel, 6-bit kernel with its automatic tile, and the
+    # 6-bit kernel's 128 x 128 tile forced (flh_gemm_set_tuning, the tests' hook).
+    cold_w = {}
+    a4q, a4s = ops.rotate_and_quantize_i4(acts["attn_in"], hadamard=had_mode(4096))
+    a11q, a11s = ops.rotate_and_quantize_i4(acts["mlp_mid"], hadamard=had_mode(11008))
+    a4q6, a11q6 = ops.encode_f6(a4q), ops.encode_f6(a11q)
+    sc4 = (torch.rand(4096, 1, device=dev) * 0.015 + 0.005).half()
+    sc11 = (torch.rand(11008, 1, device=dev) * 0.015 + 0.005).half()
+
+    def cycle_us(run, sets, reps=36):
+        at = [0]
+
+        def once():
+            at[0] = (at[0] + 1) % len(sets)
+            run(sets[at[0]])
+        for _ in range(40):
+            once()
+        torch.cuda.synchronize()
+        best = None
+        for _ in range(3):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(reps):
+                once()
+            e1.record()
+            torch.cuda.synchronize()
+            us = e0.elapsed_time(e1) * 1e3 / reps
+            best = us if best is None else min(best, us)
+        return best
+
+    rand_w = lambda n, k: torch.randint(0, 256, (n, k // 2), dtype=torch.uint8, device=dev)
+    for name, copies, shapes, k in (("qkv_one_launch", 10, [(4096, 4096)] * 3, 4096), ("o", 30, [(4096, 4096)], 4096),
+                                    ("gate_up_swiglu", 6, [(11008, 4096)] * 2, 4096), ("down", 10, [(4096, 11008)], 11008)):
+        sets8 = [[rand_w(n, kk) for n, kk in shapes] for _ in range(copies)]
+        sets6 = [[ops.encode_f6(w) for w in ws] for ws in sets8]
+        aq, a_s, aq6 = (a4q, a4s, a4q6) if k == 4096 else (a11q, a11s, a11q6)
+        scs = [sc11 if n == 11008 else sc4 for n, _ in shapes]
+        if name == "gate_up_swiglu":
+            run8 = lambda ws: ops.gemm_i4_swiglu(aq, ws[0], ws[1], a_s, scs[0], scs[1])
+            run6 = lambda ws: ops.gemm_f6_swiglu(aq6, ws[0], ws[1], a_s, scs[0], scs[1])
+        elif len(shapes) > 1:
+            run8 = lambda ws: ops.gemm_i4_dequant_multi(aq, ws, a_s, scs, -1)
+            run6 = lambda ws: ops.gemm_f6_dequant_multi(aq6, ws, a_s, scs)
+        else:
+            run8 = lambda ws: ops.gemm_i4_dequant_o16(aq, ws[0], a_s, scs[0])
+            run6 = lambda ws: ops.gemm_f6_dequant_o16(aq6, ws[0], a_s, scs[0])
+        fig = {"int8_us": round(cycle_us(run8, sets8), 1), "int8_cached_us": round(cycle_us(run8, sets8[:1]), 1),
+               "six_bit_us": round(cycle_us(run6, sets6), 1), "six_bit_cached_us": round(cycle_us(run6, sets6[:1]), 1)}
+        ops.gemm_set_tuning(128, 0)
+        fig["six_bit_128x128_tile_us"] = round(cycle_us(run6, sets6), 1)
+        fig["six_bit_128x128_tile_cached_us"] = round(cycle_us(run6, sets6[:1]), 1)
+        ops.gemm_set_tuning(0, 0)
+        fig["weight_sets"] = copies
+        cold_w[name] = fig
+        del sets8, sets6
+    del a4q6, a11q6
+
     if args.copy_calibration:
         src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).fill_(3)
         dst = torch.empty_like(src)
@@ -1142,6 +1201,7 @@ def main():
         f"llama3_8b_block_M={M},weight_groups_of_128": llama3,
         "llama3_8b_decode_linears,weight_groups_of_128": llama3_decode,
         "vendor_gemm_reference": vendor,
+        "gemm_launches_on_weights_from_hbm": cold_w,
         f"gemm_{n_act}x{k_act}_by_operand_activity": activity,
         "us_per_layer": round(ms_per_step * 1e3, 1),
         "shared_activation_launches": {"us_per_layer": round(ms_shared * 1e3, 1),
